@@ -37,8 +37,10 @@ def _run(cmd, **kw):
     if proc.returncode != 0:
         sys.stderr.write(" ".join(map(str, cmd)) + "\n" + proc.stdout + "\n")
         raise RuntimeError(f"command failed ({proc.returncode}): {cmd[0]} ... {cmd[-1]}")
-    if proc.stdout.strip():
-        sys.stderr.write(proc.stdout)
+    # hipcc's host pass does not know the device-only target feature and says so once per file
+    out = "".join(l for l in proc.stdout.splitlines(True) if "packed-fp32-ops" not in l)
+    if out.strip():
+        sys.stderr.write(out)
 
 
 def core_path() -> Path:
@@ -88,16 +90,53 @@ def build_selftest(sanitize: str = "address,undefined") -> Path:
     return out
 
 
-def build_kernels(force: bool = False, jobs: int = 8) -> Path:
+# Source groups of the kernel library. A full build links all of them; a tool that serves one
+# model family on a fresh checkout builds only what that family launches (the device runtime,
+# the GEMMs, the row kernels and the sampler are common to all). Files not listed are "transformer".
+KERNEL_GROUPS = {
+    "base": ["device_runtime.hip", "elementwise.hip", "gemm.hip", "gemm256.hip", "gemm256w.hip", "gemm_panel.hip",
+             "kgemm.hip", "sampling.hip"],
+    "hybrid": ["hybrid.hip"],
+}
+
+
+def kernel_groups_path() -> Path:
+    return NATIVE_DIR / "liblc_kernels.groups"
+
+
+def built_kernel_groups() -> set:
+    """Groups the library on disk was linked from (empty when there is none)."""
+    if not kernels_path().exists():
+        return set()
+    p = kernel_groups_path()
+    return set(p.read_text().split()) if p.exists() else {"base", "transformer", "hybrid"}
+
+
+def _group_of(name: str) -> str:
+    for g, files in KERNEL_GROUPS.items():
+        if name in files:
+            return g
+    return "transformer"
+
+
+def build_kernels(force: bool = False, jobs: int = 8, groups=None) -> Path:
+    """``groups``: the source groups to link (default: all). Objects are cached per file, so
+    widening a partial library later compiles only what is missing."""
     src_dir = ROOT / "csrc" / "kernels"
     # the device runtime (host code over the HIP runtime API) lives in the same library
     srcs = sorted(src_dir.glob("*.hip")) + sorted((ROOT / "csrc" / "runtime").glob("*.hip"))
+    all_groups = {"base", "transformer", "hybrid"}
+    groups = all_groups if groups is None else set(groups) | {"base"}
+    if groups - all_groups:
+        raise ValueError(f"unknown kernel groups {sorted(groups - all_groups)}")
+    srcs = [s for s in srcs if _group_of(s.name) in groups]
     hdrs = sorted(src_dir.glob("*.h")) + sorted(src_dir.glob("*.hpp")) + sorted(src_dir.glob("*.cuh"))
     obj_dir = BUILD_DIR / "kernels"
     obj_dir.mkdir(parents=True, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     flags = [f"--offload-arch={GFX_ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-math-errno", "-ffp-contract=fast",
-             "-fno-gpu-rdc", "-Wall", "-Wno-unused-function", f"-I{src_dir}"]
+             "-fno-gpu-rdc", "-Wall", "-Wno-unused-function", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             f"-I{src_dir}"]
     todo = []
     objs = []
     for s in srcs:
@@ -108,8 +147,11 @@ def build_kernels(force: bool = False, jobs: int = 8) -> Path:
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
         list(ex.map(_run, todo))
     out = kernels_path()
-    if force or todo or _newer_than(out, objs):
-        _run([hipcc, f"--offload-arch={GFX_ARCH}", "-shared", "-fPIC", "-o", str(out), *map(str, objs)])
+    if force or todo or _newer_than(out, objs) or built_kernel_groups() != groups:
+        tmp = out.with_suffix(".so.tmp")          # never leave a half-written library behind
+        _run([hipcc, f"--offload-arch={GFX_ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+        os.replace(tmp, out)
+        kernel_groups_path().write_text(" ".join(sorted(groups)) + "\n")
     return out
 
 

@@ -204,8 +204,8 @@ PYBIND11_MODULE(_core, m) {
       .def_readonly("blocks_free", &KVStats::blocks_free)
       .def_readonly("blocks_cached", &KVStats::blocks_cached);
   py::class_<KVManager, std::shared_ptr<KVManager>>(m, "KVManager")
-      .def(py::init<int, int, bool>(), py::arg("num_blocks"), py::arg("block_size"),
-           py::arg("enable_prefix_cache") = true)
+      .def(py::init<int, int, bool, int>(), py::arg("num_blocks"), py::arg("block_size"),
+           py::arg("enable_prefix_cache") = true, py::arg("num_state_slots") = 0)
       .def("create_sequence",
            [](KVManager& kv, i32arr tokens, bool allow_cache_hit) {
              int cached = 0;
@@ -223,6 +223,9 @@ PYBIND11_MODULE(_core, m) {
       .def("fork", &KVManager::fork)
       .def("free_sequence", &KVManager::free_sequence)
       .def("num_tokens", &KVManager::num_tokens)
+      .def("state_slot", &KVManager::state_slot)
+      .def_property_readonly("num_state_slots", &KVManager::num_state_slots)
+      .def_property_readonly("free_state_slots", &KVManager::free_state_slots)
       .def("block_table", [](const KVManager& kv, int seq) { return kv.block_table(seq); })
       .def("shared_prefix_blocks", &KVManager::shared_prefix_blocks)
       .def("take_pending_copies", &KVManager::take_pending_copies)
@@ -235,7 +238,8 @@ PYBIND11_MODULE(_core, m) {
   py::enum_<RequestKind>(m, "RequestKind")
       .value("Generate", RequestKind::Generate)
       .value("Score", RequestKind::Score)
-      .value("Embed", RequestKind::Embed);
+      .value("Embed", RequestKind::Embed)
+      .value("Replay", RequestKind::Replay);
   py::enum_<FinishReason>(m, "FinishReason")
       .value("Length", FinishReason::Length)
       .value("Eos", FinishReason::Eos)
@@ -296,6 +300,8 @@ PYBIND11_MODULE(_core, m) {
                                return a;
                              })
       .def_property_readonly("context_lens", [](const StepPlan& p) { return to_array(p.context_lens); })
+      .def_property_readonly("state_slots", [](const StepPlan& p) { return to_array(p.state_slots); })
+      .def_property_readonly("replay_order", [](const StepPlan& p) { return to_array(p.replay_order); })
       .def_property_readonly("token_ids", [](const StepPlan& p) { return to_array(p.token_ids); })
       .def_property_readonly("positions", [](const StepPlan& p) { return to_array(p.positions); })
       .def_property_readonly("slot_mapping", [](const StepPlan& p) { return to_array(p.slot_mapping); })
@@ -325,6 +331,9 @@ PYBIND11_MODULE(_core, m) {
       .def("abort_request", &Scheduler::abort_request)
       .def("schedule", &Scheduler::schedule)
       .def("schedule_ahead", &Scheduler::schedule_ahead)
+      .def("add_replay_request", &Scheduler::add_replay_request)
+      .def("schedule_replay", &Scheduler::schedule_replay)
+      .def("end_replay", &Scheduler::end_replay)
       .def("set_mix_decode", &Scheduler::set_mix_decode)
       .def_property_readonly("mix_decode", &Scheduler::mix_decode)
       .def("prefill_sample_layout", &Scheduler::prefill_sample_layout)

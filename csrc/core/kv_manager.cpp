@@ -28,9 +28,14 @@ void BlockAllocator::decref(int b) {
   if (--ref_[b] == 0) free_.push_back(b);
 }
 
-KVManager::KVManager(int num_blocks, int block_size, bool enable_prefix_cache)
-    : block_size_(block_size), prefix_cache_(enable_prefix_cache), alloc_(num_blocks) {
+KVManager::KVManager(int num_blocks, int block_size, bool enable_prefix_cache, int num_state_slots)
+    : block_size_(block_size), prefix_cache_(enable_prefix_cache), num_slots_(std::max(0, num_state_slots)),
+      alloc_(num_blocks) {
   if (block_size <= 0) throw std::invalid_argument("KVManager: block_size must be positive");
+  // A cached prefix carries keys and values but no recurrent state: the two do not combine.
+  if (num_slots_ > 0 && enable_prefix_cache)
+    throw std::invalid_argument("KVManager: state slots and the prefix cache exclude each other");
+  for (int i = num_slots_ - 1; i >= 0; --i) free_slots_.push_back(i);
 }
 
 uint64_t KVManager::hash_block(uint64_t prev, const int32_t* tok, int n) {
@@ -84,6 +89,7 @@ int KVManager::create_sequence(const int32_t* tokens, int n, int* cached_tokens,
   if (n <= 0) throw std::invalid_argument("KVManager::create_sequence: empty prompt");
   Seq s;
   int matched = 0;
+  if (num_slots_ > 0 && free_slots_.empty()) return -1;
   if (prefix_cache_ && allow_cache_hit) {
     // At least one token must be left to run so the step produces logits.
     int max_match = (n - 1) / block_size_;
@@ -107,6 +113,10 @@ int KVManager::create_sequence(const int32_t* tokens, int n, int* cached_tokens,
       return -1;
     }
     s.blocks.push_back(b);
+  }
+  if (num_slots_ > 0) {
+    s.slot = free_slots_.back();
+    free_slots_.pop_back();
   }
   s.num_tokens = matched * block_size_;
   if (cached_tokens) *cached_tokens = s.num_tokens;
@@ -203,6 +213,7 @@ void KVManager::commit(int seq, const int32_t* tokens, int n) {
 
 int KVManager::fork(int seq) {
   const Seq& src = seqs_.at(seq);
+  if (num_slots_ > 0) throw std::logic_error("KVManager::fork: sequences with a state slot cannot be forked");
   Seq s = src;
   for (int b : s.blocks) alloc_.incref(b);
   int id = next_seq_++;
@@ -223,8 +234,11 @@ void KVManager::free_sequence(int seq) {
                             pending_copies_.end());
     }
   }
+  if (it->second.slot >= 0) free_slots_.push_back(it->second.slot);
   seqs_.erase(it);
 }
+
+int KVManager::state_slot(int seq) const { return seqs_.at(seq).slot; }
 
 int KVManager::num_tokens(int seq) const { return seqs_.at(seq).num_tokens; }
 

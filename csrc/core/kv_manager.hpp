@@ -47,7 +47,13 @@ struct KVStats {
 
 class KVManager {
  public:
-  KVManager(int num_blocks, int block_size, bool enable_prefix_cache);
+  // `num_state_slots` > 0: every sequence also owns one slot of fixed-size per-sequence state
+  // (the recurrent state of models that have any; the engine owns the memory, one row per
+  // slot). A sequence takes a free slot when it is created and gives it back when it is freed;
+  // with no slot free, create_sequence fails like it does for blocks. Whoever writes a slot
+  // first (the sequence's token at position 0) starts from a zero state, so slots are not
+  // cleared here. Forked sequences cannot share a slot: fork() throws for such a manager.
+  KVManager(int num_blocks, int block_size, bool enable_prefix_cache, int num_state_slots = 0);
 
   // Creates a sequence for `tokens` (the prompt). Full leading blocks found in the
   // prefix cache are attached by reference. Returns the sequence id, or -1 if
@@ -76,6 +82,10 @@ class KVManager {
   void free_sequence(int seq);
 
   int num_tokens(int seq) const;
+  // The sequence's state slot, -1 for a manager without slots.
+  int state_slot(int seq) const;
+  int num_state_slots() const { return num_slots_; }
+  int free_state_slots() const { return static_cast<int>(free_slots_.size()); }
   const std::vector<int>& block_table(int seq) const;
   // Number of leading blocks of `seq` that are shared with at least one other
   // live sequence or the cache (refcount > 1) — the shared-prefix extent.
@@ -103,6 +113,7 @@ class KVManager {
     int num_tokens = 0;
     std::vector<uint64_t> chain;  // hash of each FULL block given its predecessors
     std::vector<int32_t> tail;    // token ids of the partially filled tail block
+    int slot = -1;                // state slot (managers with slots)
   };
   int alloc_or_evict();
   static uint64_t hash_block(uint64_t prev, const int32_t* tok, int n);
@@ -110,6 +121,8 @@ class KVManager {
 
   int block_size_;
   bool prefix_cache_;
+  int num_slots_ = 0;
+  std::vector<int> free_slots_;   // most recently freed last: a freed slot is the next one handed out
   BlockAllocator alloc_;
   std::unordered_map<int, Seq> seqs_;
   int next_seq_ = 0;

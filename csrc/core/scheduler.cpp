@@ -12,6 +12,10 @@ int Scheduler::add_request(RequestKind kind, std::vector<int32_t> prompt, int n_
                            SamplingParams p) {
   if (prompt.empty()) throw std::invalid_argument("Scheduler::add_request: empty prompt");
   if (n_chains < 1) n_chains = 1;
+  if (kind == RequestKind::Replay) throw std::invalid_argument("Scheduler::add_request: use add_replay_request");
+  // Chains fork from the prompt's sequence and would need a copy of its state slot.
+  if (n_chains > 1 && kv_->num_state_slots() > 0)
+    throw std::invalid_argument("Scheduler::add_request: a model with per-sequence state serves one chain per request");
   if (kind != RequestKind::Generate) {
     n_chains = 1;
     p.max_new_tokens = 0;
@@ -176,6 +180,9 @@ void pack_block_tables(StepPlan& plan, const KVManager& kv) {
     const auto& bt = kv.block_table(plan.seq_ids[b]);
     std::copy(bt.begin(), bt.end(), plan.block_tables.begin() + static_cast<size_t>(b) * mb);
   }
+  plan.state_slots.clear();
+  if (kv.num_state_slots() > 0)
+    for (int b = 0; b < B; ++b) plan.state_slots.push_back(kv.state_slot(plan.seq_ids[b]));
 }
 }  // namespace
 
@@ -538,9 +545,123 @@ std::vector<uint8_t> Scheduler::complete_decode(const StepPlan& plan, const int3
   return applied;
 }
 
+int Scheduler::add_replay_request() {
+  Group g;
+  g.id = next_id_++;
+  g.kind = RequestKind::Replay;
+  g.p.max_new_tokens = 0;
+  const int id = g.id;
+  groups_.emplace(id, std::move(g));
+  return id;
+}
+
+StepPlan Scheduler::schedule_replay(const std::vector<int>& request_ids,
+                                    const std::vector<std::vector<int32_t>>& tokens) {
+  if (request_ids.size() != tokens.size()) throw std::invalid_argument("schedule_replay: one token list per request");
+  const int bs = kv_->block_size();
+  const int n = static_cast<int>(request_ids.size());
+  // Everything the step needs is secured before anything is committed, so a refusal leaves the
+  // requests where they were (blocks reserved on the way stay with their sequences, unwritten).
+  std::vector<char> fresh(n, 0);
+  for (int e = 0; e < n; ++e) {
+    auto it = groups_.find(request_ids[e]);
+    if (it == groups_.end() || it->second.kind != RequestKind::Replay)
+      throw std::invalid_argument("schedule_replay: not a replayed request");
+    if (tokens[e].empty()) throw std::invalid_argument("schedule_replay: empty portion");
+    for (int f = 0; f < e; ++f)
+      if (request_ids[f] == request_ids[e]) throw std::invalid_argument("schedule_replay: a request appears twice");
+    Group& g = it->second;
+    const int take = static_cast<int>(tokens[e].size());
+    if (cfg_.max_blocks_per_seq > 0 && (g.computed + take + bs - 1) / bs > cfg_.max_blocks_per_seq)
+      throw std::invalid_argument("schedule_replay: the request outgrows the longest sequence served");
+    if (!g.admitted) {
+      int cached = 0;
+      const int seq = kv_->create_sequence(tokens[e].data(), take, &cached, false);
+      if (seq < 0) {
+        for (int f = 0; f < e; ++f)
+          if (fresh[f]) {       // give back what this call admitted
+            Group& u = groups_.at(request_ids[f]);
+            kv_->free_sequence(u.chains[0].seq);
+            u.chains.clear();
+            u.admitted = false;
+          }
+        throw std::runtime_error("schedule_replay: no blocks or no state slot for a new request");
+      }
+      g.admitted = true;
+      g.chains.assign(1, Chain{});
+      g.chains[0].seq = seq;
+      fresh[e] = 1;
+    } else if (!kv_->reserve(g.chains[0].seq, take)) {
+      for (int f = 0; f < e; ++f)
+        if (fresh[f]) {
+          Group& u = groups_.at(request_ids[f]);
+          kv_->free_sequence(u.chains[0].seq);
+          u.chains.clear();
+          u.admitted = false;
+        }
+      throw std::runtime_error("schedule_replay: the KV pool has no block for the step");
+    }
+  }
+  StepPlan plan;
+  plan.kind = StepPlan::Prefill;
+  plan.cu_q.push_back(0);
+  plan.replay_order.assign(n, -1);
+  std::vector<char> rides(n, 0);
+  for (int e = 0; e < n; ++e) rides[e] = tokens[e].size() == 1 && groups_.at(request_ids[e]).computed > 0;
+  for (int pass = 0; pass < 2; ++pass) {       // portions, then single continuation tokens
+    for (int e = 0; e < n; ++e) {
+      Group& g = groups_.at(request_ids[e]);
+      const int take = static_cast<int>(tokens[e].size());
+      const bool rider = rides[e] != 0;
+      if (rider != (pass == 1)) continue;
+      const int seq = g.chains[0].seq;
+      const auto& bt = kv_->block_table(seq);
+      const int row0 = static_cast<int>(plan.token_ids.size());
+      if (rider && plan.rider_first < 0) plan.rider_first = static_cast<int>(plan.seq_ids.size());
+      for (int i = 0; i < take; ++i) {
+        const int pos = g.computed + i;
+        plan.token_ids.push_back(tokens[e][i]);
+        plan.positions.push_back(pos);
+        plan.slot_mapping.push_back(bt[pos / bs] * bs + pos % bs);
+      }
+      plan.replay_order[e] = static_cast<int>(plan.seq_ids.size());
+      plan.seq_ids.push_back(seq);
+      plan.request_ids.push_back(g.id);
+      plan.context_lens.push_back(g.computed + take);
+      plan.cu_q.push_back(row0 + take);
+      if (rider) {
+        plan.step_index.push_back(0);
+        plan.seeds.push_back(0);
+      }
+      kv_->commit(seq, tokens[e].data(), take);
+      g.prompt.insert(g.prompt.end(), tokens[e].begin(), tokens[e].end());
+      g.computed += take;
+    }
+  }
+  auto copies = kv_->take_pending_copies();
+  for (auto& c : copies) {
+    plan.copy_src.push_back(c.first);
+    plan.copy_dst.push_back(c.second);
+  }
+  pack_block_tables(plan, *kv_);
+  return plan;
+}
+
+void Scheduler::end_replay(int request_id) {
+  auto it = groups_.find(request_id);
+  if (it == groups_.end() || it->second.kind != RequestKind::Replay) return;
+  for (auto& c : it->second.chains)
+    if (c.seq >= 0) kv_->free_sequence(c.seq);
+  groups_.erase(it);
+}
+
 void Scheduler::abort_request(int request_id) {
   auto it = groups_.find(request_id);
   if (it == groups_.end()) return;
+  if (it->second.kind == RequestKind::Replay) {
+    end_replay(request_id);
+    return;
+  }
   Group& g = it->second;
   if (!g.admitted) {
     waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), request_id), waiting_.end());

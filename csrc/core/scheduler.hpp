@@ -22,6 +22,7 @@ enum class RequestKind : uint8_t {
   Generate = 0,  // sample up to max_new_tokens per chain
   Score = 1,     // prefill only; caller reads log-probs of target ids at the last position
   Embed = 2,     // prefill only; caller reads the pooled final hidden state
+  Replay = 3,    // the caller supplies the tokens portion by portion and says which portions run together
 };
 
 struct SamplingParams {
@@ -88,6 +89,7 @@ struct StepPlan {
   std::vector<int32_t> block_tables;   // [B, max_blocks] padded with -1
   int max_blocks = 0;
   std::vector<int32_t> context_lens;   // [B] KV length visible AFTER this step's tokens are written
+  std::vector<int32_t> state_slots;    // [B] per-sequence state slot (KV managers with slots), else empty
 
   // ---- prefill ----
   std::vector<int32_t> token_ids;      // [T] flattened chunk tokens
@@ -116,6 +118,10 @@ struct StepPlan {
   bool ahead = false;
   std::vector<int32_t> src_rows;       // [B] (ahead plans only)
 
+  // Replayed steps: entry i of the call is sequence replay_order[i] of this plan (portions come
+  // first, single continuation tokens ride behind them as in any mixed step).
+  std::vector<int32_t> replay_order;
+
   // Copy-on-write block copies that must run before this step's KV writes.
   std::vector<int32_t> copy_src, copy_dst;
 };
@@ -129,6 +135,18 @@ class Scheduler {
   void abort_request(int request_id);
 
   StepPlan schedule();
+
+  // Replayed requests: a trace of token ids is fed through the engine step by step, the caller
+  // deciding what each step holds. A request is admitted (sequence, blocks, state slot) by its
+  // first portion; every later portion reserves the blocks it needs. One call = one step: a
+  // Prefill plan whose sequences are the portions of more than one token (or that start a
+  // request), followed by the single continuation tokens as riders. The tokens are committed
+  // when the plan is made, like those of any prefill plan; there is nothing to complete.
+  // Throws std::runtime_error when the pool has no blocks or no state slot for the step: replayed
+  // requests are never preempted. They are invisible to schedule() and has_work().
+  int add_replay_request();
+  StepPlan schedule_replay(const std::vector<int>& request_ids, const std::vector<std::vector<int32_t>>& tokens);
+  void end_replay(int request_id);
   // The decode step that follows `inflight` (a decode plan that has been launched and not yet
   // completed), planned without its results: every chain is assumed to go on unless it reaches
   // max_new_tokens in the step in flight. Returns an Idle plan when there is no basis for that

@@ -1,0 +1,541 @@
+// Kernels of hybrid decoder designs: an fp32 residual stream with scalar-gain RMS norms on the
+// sublayer outputs, gated recurrences whose state lives in per-sequence fp32 slots (minGRU,
+// gated linear attention), attention with separate key / value widths under a chunk or window
+// mask over a paged cache, and a shape-agnostic GEMM for the projections that the MFMA kernels
+// (gemm*.hip: bf16, K a multiple of 64) do not take, including every product of the true-fp32
+// mode. Everything a recurrence or a softmax touches is fp32; only tensors that feed the next
+// matrix product are written in the activation type (bf16 or fp32, a launch-time flag).
+//
+// A step's sequences are described by cu_q [B+1] (row ranges), positions [T] and slots [B]
+// (state slot of the sequence; < 0: padding row of a recorded step, skipped). A sequence whose
+// first row is at position 0 starts from a zero state, so slots are never cleared.
+#include "common.h"
+
+namespace {
+
+template <bool F32>
+struct Act;
+template <>
+struct Act<true> {
+  typedef float type;
+  static LC_DEVICE float load(const float* p, size_t i) { return p[i]; }
+  static LC_DEVICE void store(float* p, size_t i, float v) { p[i] = v; }
+};
+template <>
+struct Act<false> {
+  typedef bf16_t type;
+  static LC_DEVICE float load(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+  static LC_DEVICE void store(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+};
+
+LC_DEVICE float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+LC_DEVICE float siluf_(float x) { return x / (1.f + expf(-x)); }
+
+// ---------------------------------------------------------------- embedding -> fp32 stream (+ activation copy)
+template <bool EF32, bool AF32>
+__global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* __restrict__ E, float* __restrict__ x,
+                                  void* __restrict__ xa, int T, int d, int vocab, const int32_t* __restrict__ feed_tok,
+                                  const int32_t* __restrict__ feed_rows) {
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= T) return;
+  int id = ids[row];
+  if (feed_rows != nullptr) {
+    const int src = feed_rows[row];
+    if (src >= 0) id = feed_tok[src];
+  }
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const typename Act<EF32>::type* e = static_cast<const typename Act<EF32>::type*>(E) + static_cast<size_t>(id) * d;
+  typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
+  for (int c = lane; c < d; c += 64) {
+    const float v = Act<EF32>::load(e, c);
+    x[static_cast<size_t>(row) * d + c] = v;
+    if (a != nullptr) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, v);
+  }
+}
+
+// ---------------------------------------------------------------- scalar-gain RMS norm of a sublayer output
+// With y: x += y * rsqrt(mean(y^2) + eps) * gain, xa = x. Without: xa = x * rsqrt(mean(x^2) + eps) * gain.
+template <bool AF32>
+__global__ void scalar_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
+                                       float eps, void* __restrict__ xa, int T, int d) {
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= T) return;
+  float* xr = x + static_cast<size_t>(row) * d;
+  const float* src = y != nullptr ? y + static_cast<size_t>(row) * d : xr;
+  float ss = 0.f;
+  for (int c = lane; c < d; c += 64) {
+    const float v = src[c];
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float r = gain[0] / sqrtf(ss / static_cast<float>(d) + eps);
+  typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
+  for (int c = lane; c < d; c += 64) {
+    float v = src[c] * r;
+    if (y != nullptr) {
+      v += xr[c];
+      xr[c] = v;
+    }
+    if (a != nullptr) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, v);
+  }
+}
+
+template <bool AF32>
+__global__ void relu2_kernel(const float* __restrict__ y, void* __restrict__ out, long long n) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(y[i], 0.f);
+  Act<AF32>::store(static_cast<typename Act<AF32>::type*>(out), i, v * v);
+}
+
+// ---------------------------------------------------------------- minGRU
+// zxg [T, 3w]: update-gate logits | candidate pre-activations | output-gate logits.
+// One thread per (sequence, channel); the recurrence runs over the sequence's rows in order.
+template <bool AF32>
+__global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restrict__ state,
+                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                   const int32_t* __restrict__ slots, void* __restrict__ out, int w) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int slot = slots[b];
+  const int r0 = cu_q[b], r1 = cu_q[b + 1];
+  if (c >= w || slot < 0 || r1 <= r0) return;
+  float S = positions[r0] == 0 ? 0.f : state[static_cast<size_t>(slot) * w + c];
+  typename Act<AF32>::type* o = static_cast<typename Act<AF32>::type*>(out);
+  for (int t = r0; t < r1; ++t) {
+    const float* row = zxg + static_cast<size_t>(t) * 3 * w;
+    const float z = sigmoidf_(row[c]);
+    const float u = row[w + c];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
+    S = (1.f - z) * S + z * cand;
+    Act<AF32>::store(o, static_cast<size_t>(t) * w + c, S * siluf_(row[2 * w + c]));
+  }
+  state[static_cast<size_t>(slot) * w + c] = S;
+}
+
+// ---------------------------------------------------------------- gated linear attention
+// proj [T, ld]: q | k | v at columns 0, H*D, 2*H*D; decay [T, H*D] logits. One block per
+// (value-column tile of 64, head, sequence); thread dv keeps column dv of the head's state
+// S [D, Dv] in registers (DMAX >= D). Per token the block stages q, k and the decay in LDS
+// (double buffered: one barrier per token), then S = a * S + k v^T, o = S^T q.
+template <int DMAX>
+__global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ proj, int ld,
+                                                      const float* __restrict__ decay, float* __restrict__ state,
+                                                      const int32_t* __restrict__ cu_q,
+                                                      const int32_t* __restrict__ positions,
+                                                      const int32_t* __restrict__ slots, float* __restrict__ out, int H,
+                                                      int D, int Dv, float inv_tau, float qscale) {
+  __shared__ float sh[2][3][DMAX];
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int dv = blockIdx.x * 64 + threadIdx.x;
+  const int slot = slots[b];
+  const int r0 = cu_q[b], r1 = cu_q[b + 1];
+  if (slot < 0 || r1 <= r0) return;
+  const bool live = dv < Dv;
+  float S[DMAX];
+  float* st = state + (static_cast<size_t>(slot) * H + h) * D * Dv;
+  const bool fresh = positions[r0] == 0;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) S[d] = (!fresh && live && d < D) ? st[static_cast<size_t>(d) * Dv + dv] : 0.f;
+  auto stage = [&](int t, int buf) {
+    const float* row = proj + static_cast<size_t>(t) * ld + h * D;
+    const float* drow = decay + static_cast<size_t>(t) * H * D + h * D;
+    for (int d = threadIdx.x; d < D; d += 64) {
+      sh[buf][0][d] = row[d] * qscale;
+      sh[buf][1][d] = row[H * D + d];
+      const float z = drow[d];
+      // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
+      sh[buf][2][d] = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+    }
+  };
+  stage(r0, 0);
+  __syncthreads();
+  for (int t = r0; t < r1; ++t) {
+    const int buf = (t - r0) & 1;
+    if (t + 1 < r1) stage(t + 1, buf ^ 1);
+    const float v = live ? proj[static_cast<size_t>(t) * ld + 2 * H * D + h * Dv + dv] : 0.f;
+    float o = 0.f;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+      if (d < D) {
+        S[d] = sh[buf][2][d] * S[d] + sh[buf][1][d] * v;
+        o += S[d] * sh[buf][0][d];
+      }
+    }
+    if (live) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
+    __syncthreads();
+  }
+  if (live) {
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+      if (d < D) st[static_cast<size_t>(d) * Dv + dv] = S[d];
+  }
+}
+
+// Per head: o / sqrt(mean(o^2) + eps) * w, times silu(gate). One wave per (row, head).
+template <bool AF32>
+__global__ void headnorm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                     const float* __restrict__ gate, int ld_gate, void* __restrict__ out, int T, int H,
+                                     int Dv, float eps) {
+  const int idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (idx >= T * H) return;
+  const int row = idx / H, h = idx % H;
+  const float* orow = o + static_cast<size_t>(row) * H * Dv + h * Dv;
+  const float* grow = gate + static_cast<size_t>(row) * ld_gate + h * Dv;
+  float ss = 0.f;
+  for (int c = lane; c < Dv; c += 64) ss += orow[c] * orow[c];
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / static_cast<float>(Dv) + eps);
+  typename Act<AF32>::type* dst = static_cast<typename Act<AF32>::type*>(out);
+  for (int c = lane; c < Dv; c += 64)
+    Act<AF32>::store(dst, static_cast<size_t>(row) * H * Dv + h * Dv + c, orow[c] * r * w[c] * siluf_(grow[c]));
+}
+
+// ---------------------------------------------------------------- attention: norms, rotation, cache write
+// One block per token. qkv [T, ld] fp32: q [H*D] | k [G*D] | v [G*Dv]. q and k are RMS-normed over
+// their whole projection (weights qn, kn), the first rot_dims coordinates of each head rotate by
+// position * inv_freq[i] (coordinate i with i + rot_dims/2), each value head is scaled to unit RMS.
+template <bool CF32>
+__global__ __launch_bounds__(256) void qkv_prep_kernel(
+    const float* __restrict__ qkv, int ld, const float* __restrict__ qn, const float* __restrict__ kn,
+    const float* __restrict__ inv_freq, const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping,
+    void* __restrict__ kc, void* __restrict__ vc, float* __restrict__ q_out, int H, int G, int D, int Dv, int BS,
+    int rot_dims, float eps, int has_kv) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const float* row = qkv + static_cast<size_t>(t) * ld;
+  const float pos = static_cast<float>(positions[t]);
+  const int half = rot_dims >> 1;
+  const int nq = H * D, nk = G * D;
+  float ssq = 0.f, ssk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) ssq += row[i] * row[i];
+  if (has_kv)
+    for (int i = threadIdx.x; i < nk; i += blockDim.x) ssk += row[nq + i] * row[nq + i];
+  const float rq = 1.f / sqrtf(block_sum(ssq, red) / static_cast<float>(nq) + eps);
+  const float rk = has_kv ? 1.f / sqrtf(block_sum(ssk, red) / static_cast<float>(nk) + eps) : 0.f;
+  auto rotated = [&](const float* src, const float* w, float r, int idx) {
+    const int i = idx % D;
+    const float a = src[idx] * r * w[idx];
+    if (i >= rot_dims) return a;
+    const int j = i < half ? i : i - half;
+    const float ang = pos * inv_freq[j];
+    const float c = cosf(ang), s = sinf(ang);
+    if (i < half) return a * c - src[idx + half] * r * w[idx + half] * s;
+    return a * c + src[idx - half] * r * w[idx - half] * s;
+  };
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) q_out[static_cast<size_t>(t) * nq + i] = rotated(row, qn, rq, i);
+  if (!has_kv) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const size_t blk = slot / BS, off = slot % BS;
+  typename Act<CF32>::type* kd = static_cast<typename Act<CF32>::type*>(kc);
+  typename Act<CF32>::type* vd = static_cast<typename Act<CF32>::type*>(vc);
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const int g = i / D;
+    Act<CF32>::store(kd, ((blk * G + g) * BS + off) * D + (i % D), rotated(row + nq, kn, rk, i));
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const float* v = row + nq + nk;
+  for (int g = wave; g < G; g += nw) {
+    float ss = 0.f;
+    for (int c = lane; c < Dv; c += 64) ss += v[g * Dv + c] * v[g * Dv + c];
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / static_cast<float>(Dv) + eps);
+    for (int c = lane; c < Dv; c += 64) Act<CF32>::store(vd, ((blk * G + g) * BS + off) * Dv + c, v[g * Dv + c] * r);
+  }
+}
+
+// ---------------------------------------------------------------- attention over the paged cache
+// One wave per (row, query head), four heads of a row per block (same trip count for all four). Keys visible to the row at
+// position p: lo <= j <= p with lo = max(floor(p / chunk) * chunk, p - window + 1) (either limit
+// off when 0). Per tile of 64 keys: lane j scores key lo + 64 * tile + j in fp32 (q from LDS),
+// online softmax across the wave, then the lanes split the value columns and walk the tile's
+// keys (weights and cache rows from LDS). Serves prompt portions and single decoded tokens.
+constexpr int kMaxVCols = 4;   // value width up to 256
+
+template <bool CF32, bool AF32>
+__global__ __launch_bounds__(256) void attn_masked_kernel(
+    const float* __restrict__ q, const void* __restrict__ kc, const void* __restrict__ vc,
+    const int32_t* __restrict__ block_tables, int MB, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ positions, void* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale,
+    int chunk, int window) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x;
+  const bool live = blockIdx.y * 4 + wave < H;     // idle waves still take part in the barriers
+  const int h = live ? blockIdx.y * 4 + wave : H - 1;
+  float* qs = lds + wave * (D + 128);
+  float* ps = qs + D;
+  int* rows = reinterpret_cast<int*>(ps + 64);
+  const int seq = row_seq[t];
+  const int p = positions[t];
+  if (seq < 0 || p < 0) return;             // the same for every wave of the block
+  const int g = h / (H / G);
+  for (int d = lane; d < D; d += 64) qs[d] = q[(static_cast<size_t>(t) * H + h) * D + d] * scale;
+  int lo = 0;
+  if (chunk > 0) lo = (p / chunk) * chunk;
+  if (window > 0) lo = max(lo, p - window + 1);
+  const int32_t* table = block_tables + static_cast<size_t>(seq) * MB;
+  const typename Act<CF32>::type* kbase = static_cast<const typename Act<CF32>::type*>(kc);
+  const typename Act<CF32>::type* vbase = static_cast<const typename Act<CF32>::type*>(vc);
+  float m = -INFINITY, l = 0.f;
+  float acc[kMaxVCols];
+#pragma unroll
+  for (int i = 0; i < kMaxVCols; ++i) acc[i] = 0.f;
+  __syncthreads();
+  for (int j0 = lo; j0 <= p; j0 += 64) {
+    const int j = j0 + lane;
+    const bool valid = j <= p;
+    float s = -INFINITY;
+    int crow = 0;
+    if (valid) {
+      crow = (table[j / BS] * G + g) * BS + (j % BS);
+      const typename Act<CF32>::type* kr = kbase + static_cast<size_t>(crow) * D;
+      float dot = 0.f;
+      for (int d = 0; d < D; ++d) dot += qs[d] * Act<CF32>::load(kr, d);
+      s = dot;
+    }
+    const float mt = fmaxf(m, wave_max(s));
+    const float pj = valid ? expf(s - mt) : 0.f;
+    const float corr = expf(m - mt);         // exp(-inf) = 0 on the first tile
+    l = l * corr + wave_sum(pj);
+    m = mt;
+    ps[lane] = pj;
+    rows[lane] = crow;
+    __syncthreads();
+    const int n = min(64, p - j0 + 1);
+#pragma unroll
+    for (int i = 0; i < kMaxVCols; ++i) {
+      const int c = lane + 64 * i;
+      if (c < Dv) {
+        float a = acc[i] * corr;
+        for (int jj = 0; jj < n; ++jj) a += ps[jj] * Act<CF32>::load(vbase, static_cast<size_t>(rows[jj]) * Dv + c);
+        acc[i] = a;
+      }
+    }
+    __syncthreads();
+  }
+  typename Act<AF32>::type* o = static_cast<typename Act<AF32>::type*>(out);
+#pragma unroll
+  for (int i = 0; i < kMaxVCols; ++i) {
+    const int c = lane + 64 * i;
+    if (live && c < Dv) Act<AF32>::store(o, (static_cast<size_t>(t) * H + h) * Dv + c, acc[i] / l);
+  }
+}
+
+// ---------------------------------------------------------------- shape-agnostic GEMM
+// C[M, N] = A[M, K] W[N, K]^T (+ bias) with fp32 accumulation on the vector ALUs: 64 x 64 tiles,
+// 16-deep slabs in LDS, 4 x 4 outputs per thread. Any M, N, K; A, W and C each fp32 or bf16.
+// epi 1: square of relu.
+template <bool AF32, bool WF32, bool CF32>
+__global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ A, const void* __restrict__ W,
+                                                       const void* __restrict__ bias, void* __restrict__ C, int M, int N,
+                                                       int K, int epi) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A);
+  const typename Act<WF32>::type* w = static_cast<const typename Act<WF32>::type*>(W);
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    for (int i = threadIdx.x; i < 64 * 16; i += 256) {
+      const int r = i >> 4, k = i & 15;
+      As[k][r] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * K + k0 + k) : 0.f;
+      Ws[k][r] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        av[i] = As[k][ty * 4 + i];
+        wv[i] = Ws[k][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * wv[j];
+    }
+    __syncthreads();
+  }
+  typename Act<CF32>::type* c = static_cast<typename Act<CF32>::type*>(C);
+  const typename Act<WF32>::type* bs = static_cast<const typename Act<WF32>::type*>(bias);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = m0 + ty * 4 + i;
+    if (r >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + tx * 4 + j;
+      if (col >= N) continue;
+      float v = acc[i][j] + (bs != nullptr ? Act<WF32>::load(bs, col) : 0.f);
+      if (epi == 1) {
+        v = fmaxf(v, 0.f);
+        v *= v;
+      }
+      Act<CF32>::store(c, static_cast<size_t>(r) * N + col, v);
+    }
+  }
+}
+
+}  // namespace
+
+// ================================================================= launchers
+LC_EXPORT int lc_embed_rows(const void* ids, const void* E, int e_f32, void* x, void* xa, int act_f32, int T, int d,
+                            int vocab, const void* feed_tok, const void* feed_rows, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (d <= 0 || vocab <= 0) return -1;
+  const dim3 grid((T + 3) / 4), block(256);
+#define LC_EMB(E32, A32)                                                                                      \
+  embed_rows_kernel<E32, A32><<<grid, block, 0, st>>>(static_cast<const int32_t*>(ids), E, static_cast<float*>(x), \
+                                                      xa, T, d, vocab, static_cast<const int32_t*>(feed_tok), \
+                                                      static_cast<const int32_t*>(feed_rows))
+  if (e_f32 && act_f32) LC_EMB(true, true);
+  else if (e_f32) LC_EMB(true, false);
+  else if (act_f32) LC_EMB(false, true);
+  else LC_EMB(false, false);
+#undef LC_EMB
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_scalar_norm_add(void* x, const void* y, const void* gain, float eps, void* xa, int act_f32, int T,
+                                 int d, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (d <= 0) return -1;
+  const dim3 grid((T + 3) / 4), block(256);
+  if (act_f32)
+    scalar_norm_add_kernel<true><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y),
+                                                         static_cast<const float*>(gain), eps, xa, T, d);
+  else
+    scalar_norm_add_kernel<false><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y),
+                                                          static_cast<const float*>(gain), eps, xa, T, d);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_relu2(const void* y, void* out, int act_f32, long long n, hipStream_t st) {
+  if (n <= 0) return 0;
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256)), block(256);
+  if (act_f32) relu2_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n);
+  else relu2_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_mingru_scan(const void* zxg, void* state, const void* cu_q, const void* positions, const void* slots,
+                             void* out, int act_f32, int B, int w, hipStream_t st) {
+  if (B <= 0) return 0;
+  if (w <= 0) return -1;
+  const dim3 grid((w + 127) / 128, B), block(128);
+  if (act_f32)
+    mingru_scan_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(zxg), static_cast<float*>(state),
+                                                     static_cast<const int32_t*>(cu_q),
+                                                     static_cast<const int32_t*>(positions),
+                                                     static_cast<const int32_t*>(slots), out, w);
+  else
+    mingru_scan_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(zxg), static_cast<float*>(state),
+                                                      static_cast<const int32_t*>(cu_q),
+                                                      static_cast<const int32_t*>(positions),
+                                                      static_cast<const int32_t*>(slots), out, w);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* state, const void* cu_q,
+                          const void* positions, const void* slots, void* out, int B, int H, int D, int Dv, float tau,
+                          hipStream_t st) {
+  if (B <= 0) return 0;
+  if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + H * Dv || !(tau > 0.f)) return -1;
+  const dim3 grid((Dv + 63) / 64, H, B), block(64);
+  const float qscale = 1.f / sqrtf(static_cast<float>(D));
+#define LC_GLA(DMAX)                                                                                                \
+  gla_scan_kernel<DMAX><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, static_cast<const float*>(decay), \
+                                                static_cast<float*>(state), static_cast<const int32_t*>(cu_q),      \
+                                                static_cast<const int32_t*>(positions),                             \
+                                                static_cast<const int32_t*>(slots), static_cast<float*>(out), H, D, \
+                                                Dv, 1.f / tau, qscale)
+  if (D <= 32) LC_GLA(32);
+  else if (D <= 64) LC_GLA(64);
+  else if (D <= 128) LC_GLA(128);
+  else LC_GLA(256);
+#undef LC_GLA
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_headnorm_gate(const void* o, const void* w, const void* gate, int ld_gate, void* out, int act_f32,
+                               int T, int H, int Dv, float eps, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || Dv <= 0 || ld_gate < H * Dv) return -1;
+  const dim3 grid((T * H + 3) / 4), block(256);
+  if (act_f32)
+    headnorm_gate_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(o), static_cast<const float*>(w),
+                                                       static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps);
+  else
+    headnorm_gate_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(o), static_cast<const float*>(w),
+                                                        static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_qkv_prep(const void* qkv, int ld, const void* qn, const void* kn, const void* inv_freq,
+                          const void* positions, const void* slot_mapping, void* kc, void* vc, int cache_f32,
+                          void* q_out, int T, int H, int G, int D, int Dv, int BS, int rot_dims, float eps, int has_kv,
+                          hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || G <= 0 || D <= 0 || Dv <= 0 || BS <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1)) return -1;
+  if (ld < H * D + (has_kv ? G * (D + Dv) : 0)) return -1;
+  if (has_kv && (kc == nullptr || vc == nullptr || kn == nullptr)) return -1;
+#define LC_PREP(C32)                                                                                              \
+  qkv_prep_kernel<C32><<<dim3(T), dim3(256), 0, st>>>(                                                            \
+      static_cast<const float*>(qkv), ld, static_cast<const float*>(qn), static_cast<const float*>(kn),           \
+      static_cast<const float*>(inv_freq), static_cast<const int32_t*>(positions),                                \
+      static_cast<const int32_t*>(slot_mapping), kc, vc, static_cast<float*>(q_out), H, G, D, Dv, BS, rot_dims, eps, \
+      has_kv)
+  if (cache_f32) LC_PREP(true);
+  else LC_PREP(false);
+#undef LC_PREP
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int cache_f32, const void* block_tables,
+                             int MB, const void* row_seq, const void* positions, void* out, int act_f32, int T, int H,
+                             int G, int D, int Dv, int BS, float scale, int chunk, int window, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * kMaxVCols || BS <= 0 || MB <= 0) return -1;
+  const size_t lds = 4 * static_cast<size_t>(D + 128) * sizeof(float);
+  if (lds > 64 * 1024) return -1;
+  const dim3 grid(T, (H + 3) / 4), block(256);
+#define LC_ATT(C32, A32)                                                                                        \
+  attn_masked_kernel<C32, A32><<<grid, block, lds, st>>>(                                                       \
+      static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \
+      static_cast<const int32_t*>(row_seq), static_cast<const int32_t*>(positions), out, H, G, D, Dv, BS, scale, \
+      chunk, window)
+  if (cache_f32 && act_f32) LC_ATT(true, true);
+  else if (cache_f32) LC_ATT(true, false);
+  else if (act_f32) LC_ATT(false, true);
+  else LC_ATT(false, false);
+#undef LC_ATT
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_gemm_any(const void* A, int a_f32, const void* W, int w_f32, const void* bias, void* C, int c_f32,
+                          int M, int N, int K, int epi, hipStream_t st) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0) return -1;
+  const dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+#define LC_GA(A32, W32, C32) gemm_any_kernel<A32, W32, C32><<<grid, block, 0, st>>>(A, W, bias, C, M, N, K, epi)
+  const int sel = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
+  switch (sel) {
+    case 0: LC_GA(false, false, false); break;
+    case 1: LC_GA(false, false, true); break;
+    case 2: LC_GA(false, true, false); break;
+    case 3: LC_GA(false, true, true); break;
+    case 4: LC_GA(true, false, false); break;
+    case 5: LC_GA(true, false, true); break;
+    case 6: LC_GA(true, true, false); break;
+    default: LC_GA(true, true, true); break;
+  }
+#undef LC_GA
+  LC_RETURN_LAST_ERROR();
+}

@@ -46,6 +46,26 @@ def kernels_path() -> Path:
     return _HERE / "liblc_kernels.so"
 
 
+def ensure_kernels(groups) -> None:
+    """Makes sure the kernel library on disk holds the given source groups (build_native.py:
+    base, transformer, hybrid), building what is missing with hipcc. For tools that must work on
+    a fresh checkout; call it before the library is first loaded in the process."""
+    import sys
+
+    sys.path.insert(0, str(_ROOT))
+    try:
+        import build_native
+
+        have = build_native.built_kernel_groups()
+        need = set(groups) | {"base"}
+        if not need <= have:
+            if _KERNELS is not None:
+                raise KernelLibraryMissing(f"the loaded kernel library lacks {sorted(need - have)}")
+            build_native.build_kernels(groups=have | need, jobs=min(16, os.cpu_count() or 1))
+    finally:
+        sys.path.pop(0)
+
+
 def kernels() -> ctypes.CDLL:
     """ctypes handle of liblc_kernels.so. Raises loudly when the library is absent:
     GPU code paths never fall back to PyTorch ops."""

@@ -21,6 +21,7 @@ import torch
 from .. import ops
 from .. import runtime as rt
 from .._native import core
+from ..models.hybrid import StepLayout
 from ..models.transformer import AttnMeta, KVCache, TransformerModel
 from ..utils.log import get_logger
 from ..utils.trace import span
@@ -97,7 +98,7 @@ class _DecodeGraph:
         fields = [("seeds", 2 * B), ("token_ids", B), ("positions", B), ("slot_mapping", B), ("ctx_lens", B),
                   ("top_k", B), ("steps", B), ("kv_begin", B), ("src_rows", B), ("temperature", B), ("top_p", B),
                   ("decision_ids", B * C), ("group_first", G), ("group_count", G), ("group_shared", G),
-                  ("block_tables", B * MB)]
+                  ("block_tables", B * MB), ("state_slots", B), ("row_seq", B), ("cu_rows", B + 1)]
         total = sum(n for _, n in fields)
         if dev.type == "cuda":
             # device block and pinned host mirror from the engine's runtime arenas
@@ -126,6 +127,9 @@ class _DecodeGraph:
             self.h[name] = hv
             off += n
         self.h["slot_mapping"][:] = -1
+        self.h["state_slots"][:] = -1          # padding rows touch no sequence's state
+        self.h["row_seq"][:] = -1
+        self.h["cu_rows"][:] = np.arange(B + 1, dtype=np.int32)     # one row per sequence
         self.h["src_rows"][:] = -1
         self.h["top_p"][:] = 1.0
         self.feed_set = False                 # the mirror's src_rows hold something other than -1
@@ -173,7 +177,12 @@ class _DecodeGraph:
             self.arena.copy_(self.host)
 
     def meta(self, eng: "Engine") -> AttnMeta:
+        layout = None
+        if eng.model.wants_layout:
+            layout = StepLayout(self.cu_rows, self.row_seq, self.block_tables,
+                                self.state_slots if eng.kvm.num_state_slots else None)
         return AttnMeta(
+            layout=layout,
             is_prefill=False, block_tables=self.block_tables, ctx_lens=self.ctx_lens, nsplit=self.nsplit,
             groups=(self.group_first, self.group_count, self.group_shared) if self.with_prefix else None,
             kv_begin=self.kv_begin if self.with_prefix else None,
@@ -527,7 +536,11 @@ class Engine:
                  kv_fraction: float = 0.6, enable_prefix_cache: bool = True, use_graphs: Optional[bool] = None,
                  graph_buckets: Sequence[int] = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512), max_decision: int = 8,
                  max_group_rows: int = 16, name: str = "engine", mix_decode: bool = True,
-                 optimistic_admission: bool = False, pipeline_decode: Optional[bool] = None) -> None:
+                 optimistic_admission: bool = False, pipeline_decode: Optional[bool] = None,
+                 state_slots: Optional[int] = None) -> None:
+        """``state_slots``: how many sequences with recurrent state can be live at once (models
+        that have any; default: ``max_batch_seqs``). The KV manager hands the slots out with the
+        blocks; a model without state gets none."""
         self.model, self.device, self.name = model, model.device, name
         cfg = model.cfg
         self.block_size = block_size
@@ -537,7 +550,7 @@ class Engine:
         own_stream = self.device.type == "cuda" and not serialize_streams()
         self.rt = rt.DeviceRuntime(self.device, own_stream) if self.device.type == "cuda" else None
         if num_kv_blocks is None:
-            per_block = KVCache.bytes_per_block(cfg, block_size, model.hkv)
+            per_block = model.cache_bytes_per_block(block_size)
             if self.rt is not None:
                 with torch.cuda.device(self.rt.device):
                     free, _ = rt.mem_info()
@@ -548,8 +561,10 @@ class Engine:
         if self.rt is not None:
             def kv_alloc(numel: int) -> torch.Tensor:
                 return self.rt.reserve_kv(2 * numel + 256).tensor((numel,), torch.bfloat16)
-        self.kv = KVCache(cfg, num_kv_blocks, block_size, self.device, model.hkv, alloc=kv_alloc)
-        self.kvm = core.KVManager(num_kv_blocks, block_size, enable_prefix_cache)
+        n_slots = model.state_slots_needed(max_batch_seqs if state_slots is None else state_slots)
+        self.kv = model.make_cache(num_kv_blocks, block_size, n_slots, alloc=kv_alloc)
+        # a cached prefix holds keys and values but no recurrent state: models with state recompute
+        self.kvm = core.KVManager(num_kv_blocks, block_size, enable_prefix_cache and n_slots == 0, n_slots)
         sc = core.SchedulerConfig()
         sc.max_batch_seqs, sc.max_prefill_tokens = max_batch_seqs, max_prefill_tokens
         # Mixed steps: chains that are already decoding ride along in the steps that prefill newly
@@ -661,6 +676,8 @@ class Engine:
                                  f"{int(arr.min())} .. {int(arr.max())}")
         if n < 1:
             raise ValueError(f"n = {n}: a request has at least one chain")
+        if kind == core.RequestKind.Embed and not self.model.supports_embed:
+            raise ValueError(f"{self.name}: this model family serves no pooled embeddings")
         new = p.max_new_tokens if kind == core.RequestKind.Generate else 0
         if kind == core.RequestKind.Generate and not 1 <= new < self.max_model_len:
             raise ValueError(f"max_new_tokens = {new} must lie in [1, {self.max_model_len - 1}]: the longest sequence "
@@ -926,9 +943,7 @@ class Engine:
         # ---- everything the step reads from the host goes into one staging buffer ----
         sg = self._staging
         sg.begin()
-        t_tok, t_pos, t_slot = sg.put(plan.token_ids), sg.put(plan.positions), sg.put(plan.slot_mapping)
-        t_bt, t_ctx = sg.put(plan.block_tables), sg.put(plan.context_lens)
-        t_cu = sg.put(cu[:rf + 1] if n_riders else cu)
+        t_in = self._stage_step_inputs(plan, sg)
         # Embed requests: one pooling launch over the chunks of all of them in this step (fp32
         # sums of the final hidden states per chunk); a prompt cut into several chunks adds its
         # chunk sums up, the mean and the L2 normalisation happen when the request finishes.
@@ -986,19 +1001,7 @@ class Engine:
         # log-probs instead of all-gathering the logits rows.
         score_only = bool(want) and t_samp is None and m.tp_size > 1
         sg.ship()
-        bt, ctx = sg.view(t_bt), sg.view(t_ctx)
-        if n_riders:
-            # Mixed step: sequences [rf, n_seq) are decoding chains with one token each.
-            riders = AttnMeta(is_prefill=False, block_tables=bt[rf:], ctx_lens=ctx[rf:],
-                              nsplit=ops.choose_kv_splits(n_riders, m.hkv, int(plan.context_lens[rf:].max()))
-                              if self.device.type == "cuda" else 1)
-            meta = AttnMeta(is_prefill=True, block_tables=bt[:rf], ctx_lens=ctx[:rf], cu_q=sg.view(t_cu),
-                            max_q_len=int(np.diff(cu[:rf + 1]).max()), riders=riders, prefill_tokens=int(cu[rf]))
-            self.metrics.inc("prefill.rider_tokens", n_riders)
-        else:
-            meta = AttnMeta(is_prefill=True, block_tables=bt, ctx_lens=ctx, cu_q=sg.view(t_cu),
-                            max_q_len=int(np.diff(cu).max()))
-        hidden = m.forward(sg.view(t_tok), sg.view(t_pos), sg.view(t_slot), meta, self.kv)
+        hidden = self._run_staged_step(plan, sg, t_in)
         if emb:
             sums = ops.embed_pool_ranges(hidden, sg.view(t_eb), sg.view(t_ee), mode=2)
             for j, i in enumerate(emb):
@@ -1031,6 +1034,105 @@ class Engine:
                     k_rdec = land.take(ops.logprob_gather(logits, sg.view(rider_dec[2]), sg.view(rider_dec[1])))
         land.mark()
         return land, k_tok, k_lp, (want, k_want), (rider_dec[0] if rider_dec is not None else None, k_rdec)
+
+    def _stage_step_inputs(self, plan, sg) -> dict:
+        """Puts what the model's forward reads of a prefill-kind plan (prompt portions, possibly
+        with riders behind them) into the step's staging buffer; returns the tickets."""
+        rf, cu = plan.rider_first, plan.cu_q
+        n_riders = len(plan.seq_ids) - rf if rf >= 0 else 0
+        t = {"tok": sg.put(plan.token_ids), "pos": sg.put(plan.positions), "slot": sg.put(plan.slot_mapping),
+             "bt": sg.put(plan.block_tables), "ctx": sg.put(plan.context_lens),
+             "cu": sg.put(cu[:rf + 1] if n_riders else cu)}
+        if self.model.wants_layout:
+            # every sequence of the step in one description: row ranges, row -> sequence, state slots
+            t["cu_all"] = sg.put(cu) if n_riders else t["cu"]
+            t["row_seq"] = sg.put(np.repeat(np.arange(len(plan.seq_ids), dtype=np.int32), np.diff(cu)).astype(np.int32))
+            if len(plan.state_slots):
+                t["slots"] = sg.put(plan.state_slots)
+        return t
+
+    def _run_staged_step(self, plan, sg, t: dict, taps: Optional[list] = None) -> torch.Tensor:
+        """The model's forward over a staged prefill-kind plan (after ``sg.ship()``)."""
+        m = self.model
+        rf, cu = plan.rider_first, plan.cu_q
+        n_seq = len(plan.seq_ids)
+        n_riders = n_seq - rf if rf >= 0 else 0
+        bt, ctx = sg.view(t["bt"]), sg.view(t["ctx"])
+        layout = None
+        if m.wants_layout:
+            layout = StepLayout(sg.view(t["cu_all"]), sg.view(t["row_seq"]), bt,
+                                sg.view(t["slots"]) if "slots" in t else None)
+        if n_riders:
+            # Mixed step: sequences [rf, n_seq) are decoding chains with one token each.
+            riders = AttnMeta(is_prefill=False, block_tables=bt[rf:], ctx_lens=ctx[rf:],
+                              nsplit=ops.choose_kv_splits(n_riders, m.hkv, int(plan.context_lens[rf:].max()))
+                              if self.device.type == "cuda" else 1)
+            meta = AttnMeta(is_prefill=True, block_tables=bt[:rf], ctx_lens=ctx[:rf], cu_q=sg.view(t["cu"]),
+                            max_q_len=int(np.diff(cu[:rf + 1]).max()) if rf > 0 else 0, riders=riders,
+                            prefill_tokens=int(cu[rf]), layout=layout)
+            self.metrics.inc("prefill.rider_tokens", n_riders)
+        else:
+            meta = AttnMeta(is_prefill=True, block_tables=bt, ctx_lens=ctx, cu_q=sg.view(t["cu"]),
+                            max_q_len=int(np.diff(cu).max()), layout=layout)
+        kw = {"taps": taps} if taps is not None else {}
+        return m.forward(sg.view(t["tok"]), sg.view(t["pos"]), sg.view(t["slot"]), meta, self.kv, **kw)
+
+    # ------------------------------------------------------------------ replayed traces
+    def replay_open(self) -> int:
+        """A request whose tokens the caller supplies step by step (``replay_step``). It takes its
+        sequence, blocks and state slot with its first portion and keeps them until ``replay_close``."""
+        return self.sched.add_replay_request()
+
+    def replay_close(self, rid: int) -> None:
+        self.sched.end_replay(rid)
+
+    def replay_step(self, entries, taps: Optional[list] = None) -> np.ndarray:
+        """Runs ONE engine step over given tokens: ``entries`` = [(request, tokens, want)], every
+        request's next tokens and the places among them whose logits are asked for. Portions of
+        several tokens run as prompt portions, single continuation tokens ride behind them as
+        decoded tokens do in any mixed step; all of it is one batch through the model's forward,
+        the engine's cache and state slots. Returns fp32 logits [wanted, vocab] in the order of
+        the entries and of their wants. Nothing is sampled."""
+        if self._ahead is not None:
+            raise RuntimeError("replay_step while a decode step launched ahead is in flight")
+        vocab = self.model.cfg.vocab_size
+        toks = [np.asarray(e[1], dtype=np.int32) for e in entries]
+        for a in toks:
+            if a.size == 0 or int(a.min()) < 0 or int(a.max()) >= vocab:
+                raise ValueError(f"replay_step: empty portion or token id outside the vocabulary of {vocab}")
+        plan = self.sched.schedule_replay([int(e[0]) for e in entries], [a.tolist() for a in toks])
+        cu, order = plan.cu_q, plan.replay_order
+        need = []
+        for i, e in enumerate(entries):
+            n = len(toks[i])
+            for w in e[2]:
+                if not 0 <= int(w) < n:
+                    raise ValueError("replay_step: a wanted place lies outside its portion")
+                need.append(int(cu[int(order[i])]) + int(w))
+        with self._on_stream():
+            if len(plan.copy_src):
+                self._copy_blocks(plan.copy_src, plan.copy_dst)
+            sg = self._staging
+            sg.begin()
+            t_in = self._stage_step_inputs(plan, sg)
+            t_need = sg.put(np.asarray(need, dtype=np.int32)) if need else None
+            sg.ship()
+            hidden = self._run_staged_step(plan, sg, t_in, taps)
+            land = self._landing[self._step_no & 1]
+            land.begin()
+            k = None
+            if need:
+                logits = self.model.logits(ops.gather_rows(hidden, sg.view(t_need)))
+                land.reserve(logits.numel() * 4 + 256)
+                k = land.take(logits)
+            land.mark()
+            self._step_no += 1
+            land.wait()
+            self.metrics.inc("replay.steps")
+            self.metrics.inc("replay.tokens", len(plan.token_ids))
+            if k is None:
+                return np.zeros((0, vocab), dtype=np.float32)
+            return np.array(land.get(k), copy=True).reshape(len(need), -1)[:, :vocab]
 
     def _score_wants(self, plan) -> list:
         """(index into the step's last rows, request state, target ids) of every prompt that ends
@@ -1170,6 +1272,10 @@ class Engine:
         put("positions", plan.positions)
         put("slot_mapping", plan.slot_mapping, -1)
         put("ctx_lens", plan.context_lens)
+        if self.model.wants_layout:
+            put("row_seq", np.arange(B, dtype=np.int32), -1)
+            if len(plan.state_slots):
+                put("state_slots", plan.state_slots, -1)
         if plan.ahead:
             # the input tokens are still being sampled: row b reads last_tokens[src_rows[b]]
             put("src_rows", plan.src_rows, -1)

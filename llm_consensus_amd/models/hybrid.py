@@ -1,0 +1,531 @@
+"""Hybrid decoders: a stack whose layers each pick one mixer -- chunk-masked attention over the
+paged cache, minGRU, or gated linear attention -- around an fp32 residual stream.
+
+The design served here is Nidozen. Its ``config.json`` lists the layers (``layers[i].type``,
+``.mixer`` sizes, ``.mlp``), and every size and constant comes from there or from a tensor's shape:
+
+* a layer computes ``x += norm1(mixer(x))`` and, if it has a feed-forward, ``x += norm2(ff(x))``:
+  the sublayers read the stream itself and the norm (RMS with ONE gain for all coordinates) sits
+  on their output;
+* ``attention``: biased q/k/v/o projections, an RMS norm over the whole query (key) projection
+  before the heads are split, rotary positions on the first ``rot.dims`` coordinates of each head,
+  value heads scaled to unit RMS, grouped key/value heads of widths ``dim`` / ``vdim``, softmax over
+  the keys of the row's own chunk of ``mask.size`` positions; ``kv_from: j`` reads layer j's cache;
+* ``mingru``: S <- (1 - z) S + z c with gates that read only the current token;
+* ``gla``: per head S <- diag(a) S + k v^T, read out with q, normed per head and gated;
+* feed-forward: down(relu(up(x))^2).
+
+The residual stream, norms, scores, recurrences and their states are fp32 whatever the activation
+type (``dtype``: bf16 products with fp32 accumulation, or fp32 throughout). Keys / values live in
+the paged pool the engine's KV manager hands out blocks of; recurrent states live in per-sequence
+slots of the same manager (``HybridCache``). The step description is the engine's ``AttnMeta``
+with its ``layout`` (row ranges, row -> sequence, state slots, block tables of ALL sequences of
+the step, prompt portions and single decoded tokens alike).
+"""
+from __future__ import annotations
+
+import json
+import zlib
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .. import ops
+
+ARCHITECTURE = "Nidozen"
+MIXERS = ("attention", "mingru", "gla")
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    type: str
+    # attention / gla
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    scale: float = 0.0
+    chunk: int = 0               # keys visible only inside the row's chunk of this many positions (0: all)
+    window: int = 0              # keys visible only this far back (0: all)
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    kv_from: int = -1            # attention: read this layer's keys and values (-1: own)
+    # gla
+    tau: float = 1.0
+    rank: int = 0                # width of the decay's low-rank bottleneck (from the tensor's shape)
+    # mingru
+    width: int = 0
+    # feed-forward (0: none)
+    ff: int = 0
+
+    @property
+    def owns_kv(self) -> bool:
+        return self.type == "attention" and self.kv_from < 0
+
+    def state_size(self) -> int:
+        """fp32 numbers of recurrent state per sequence."""
+        if self.type == "mingru":
+            return self.width
+        if self.type == "gla":
+            return self.heads * self.dim * self.vdim
+        return 0
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    name: str
+    vocab_size: int
+    hidden_size: int
+    rms_eps: float
+    layers: Tuple[LayerSpec, ...]
+    max_position: int = 1 << 20
+    model_type: str = "nidozen"
+    architecture: str = ARCHITECTURE
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def has_state(self) -> bool:
+        return any(l.state_size() for l in self.layers)
+
+    @property
+    def num_heads(self) -> int:
+        return max([l.heads for l in self.layers if l.type == "attention"] or [1])
+
+    @property
+    def num_kv_heads(self) -> int:
+        return max([l.kv_heads for l in self.layers if l.type == "attention"] or [1])
+
+    def kv_elems_per_token(self) -> int:
+        return sum(l.kv_heads * (l.dim + l.vdim) for l in self.layers if l.owns_kv)
+
+    def state_floats(self) -> int:
+        return sum(l.state_size() for l in self.layers)
+
+    def param_count(self) -> int:
+        return sum(_numel(s) for s in param_shapes(self).values())
+
+    def weight_bytes(self, bytes_per_param: int = 2) -> int:
+        return self.param_count() * bytes_per_param
+
+    def validate(self) -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
+            raise ValueError(f"{self.name}: vocab, width and at least one layer are needed")
+        for i, l in enumerate(self.layers):
+            if l.type not in MIXERS:
+                raise ValueError(f"{self.name}: layer {i}: unknown mixer {l.type!r} (known: {', '.join(MIXERS)})")
+            if l.type == "mingru" and l.width <= 0:
+                raise ValueError(f"{self.name}: layer {i}: minGRU needs a width")
+            if l.type in ("attention", "gla") and (l.heads <= 0 or l.dim <= 0 or l.vdim <= 0):
+                raise ValueError(f"{self.name}: layer {i}: heads, dim and vdim are needed")
+            if l.type == "gla" and (l.dim > 256 or not l.tau > 0):
+                raise ValueError(f"{self.name}: layer {i}: gated linear attention takes dim <= 256 and tau > 0")
+            if l.type == "attention":
+                if l.kv_heads <= 0 or l.heads % l.kv_heads:
+                    raise ValueError(f"{self.name}: layer {i}: heads must be a multiple of kv_heads")
+                if l.rot_dims % 2 or l.rot_dims > l.dim:
+                    raise ValueError(f"{self.name}: layer {i}: rot.dims must be even and at most dim")
+                if l.vdim > 256:
+                    raise ValueError(f"{self.name}: layer {i}: the attention kernel takes vdim <= 256")
+                if l.kv_from >= 0:
+                    src = self.layers[l.kv_from] if l.kv_from < i else None
+                    if src is None or not src.owns_kv:
+                        raise ValueError(f"{self.name}: layer {i}: kv_from must name an earlier attention layer "
+                                         f"with keys of its own")
+                    if (src.kv_heads, src.dim, src.vdim) != (l.kv_heads, l.dim, l.vdim):
+                        raise ValueError(f"{self.name}: layer {i}: kv_from layer {l.kv_from} has other head sizes")
+
+
+def _numel(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+def config_from_dict(c: dict, name: str = "nidozen", tensor_shapes: Optional[Dict[str, tuple]] = None) -> HybridConfig:
+    """Parses a Nidozen ``config.json``. ``tensor_shapes`` (name -> shape of the checkpoint's
+    tensors) supplies the sizes the configuration leaves to the tensors."""
+    if c.get("architecture") != ARCHITECTURE:
+        raise ValueError(f"{name}: architecture {c.get('architecture')!r} is not {ARCHITECTURE}")
+    layers = []
+    for i, L in enumerate(c["layers"]):
+        t, m = L["type"], L.get("mixer") or {}
+        mlp = L.get("mlp")
+        ff = 0
+        if mlp is not None:
+            if mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"{name}: layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported")
+            ff = int(mlp["ff"])
+        if t == "attention":
+            mask, rot = m.get("mask") or {}, m.get("rot") or {}
+            kvf = m.get("kv_from")
+            layers.append(LayerSpec(t, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                                    chunk=int(mask.get("size", 0)), window=int(mask.get("window", 0)),
+                                    rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                                    kv_from=-1 if kvf is None else int(kvf), ff=ff))
+        elif t == "mingru":
+            layers.append(LayerSpec(t, width=int(m["width"]), ff=ff))
+        elif t == "gla":
+            rank = int(m.get("rank", 0))
+            if tensor_shapes is not None and f"l{i}.mix.a1" in tensor_shapes:
+                rank = int(tensor_shapes[f"l{i}.mix.a1"][0])
+            layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                    tau=float(m["tau"]), rank=rank or 16, ff=ff))
+        else:
+            raise ValueError(f"{name}: layer {i}: unknown mixer {t!r} (known: {', '.join(MIXERS)})")
+    cfg = HybridConfig(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                       rms_eps=float(c["norm"]["eps"]), layers=tuple(layers),
+                       max_position=int(c.get("max_position", 1 << 20)))
+    cfg.validate()
+    return cfg
+
+
+def config_to_dict(cfg: HybridConfig) -> dict:
+    layers = []
+    for l in cfg.layers:
+        if l.type == "attention":
+            m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                 "mask": {"size": l.chunk} if not l.window else {"size": l.chunk, "window": l.window},
+                 "rot": {"dims": l.rot_dims, "base": l.rot_base}}
+            if l.kv_from >= 0:
+                m["kv_from"] = l.kv_from
+        elif l.type == "mingru":
+            m = {"width": l.width}
+        else:
+            m = {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "tau": l.tau, "rank": l.rank}
+        layers.append({"type": l.type, "mixer": m, "mlp": {"kind": "dense", "ff": l.ff} if l.ff else None})
+    return {"architecture": ARCHITECTURE, "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "norm": {"eps": cfg.rms_eps}, "layers": layers}
+
+
+def config_from_path(path: str) -> HybridConfig:
+    p = Path(path)
+    d = p if p.is_dir() else p.parent
+    c = json.loads((d / "config.json").read_text())
+    shapes = None
+    st = d / "model.safetensors"
+    if st.exists():
+        from safetensors import safe_open
+
+        with safe_open(str(st), framework="pt", device="cpu") as h:
+            shapes = {k: tuple(h.get_slice(k).get_shape()) for k in h.keys()}
+    return config_from_dict(c, name=d.name, tensor_shapes=shapes)
+
+
+def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
+    """Checkpoint tensor names -> shapes (linear weights are [out, in])."""
+    d = cfg.hidden_size
+    out: Dict[str, tuple] = {"embed": (cfg.vocab_size, d)}
+    for i, l in enumerate(cfg.layers):
+        p = f"l{i}."
+        out[p + "norm1"] = ()
+        if l.ff:
+            out[p + "norm2"] = ()
+        m = p + "mix."
+        if l.type == "attention":
+            out[m + "q"], out[m + "q.b"], out[m + "q.norm"] = (l.heads * l.dim, d), (l.heads * l.dim,), (l.heads * l.dim,)
+            if l.owns_kv:
+                out[m + "k"], out[m + "k.b"] = (l.kv_heads * l.dim, d), (l.kv_heads * l.dim,)
+                out[m + "k.norm"] = (l.kv_heads * l.dim,)
+                out[m + "v"], out[m + "v.b"] = (l.kv_heads * l.vdim, d), (l.kv_heads * l.vdim,)
+            out[m + "o"], out[m + "o.b"] = (d, l.heads * l.vdim), (d,)
+        elif l.type == "mingru":
+            for n in ("z", "x", "g"):
+                out[m + n] = (l.width, d)
+            out[m + "z.b"], out[m + "x.b"] = (l.width,), (l.width,)
+            out[m + "o"] = (d, l.width)
+        else:
+            out[m + "q"], out[m + "k"] = (l.heads * l.dim, d), (l.heads * l.dim, d)
+            out[m + "v"], out[m + "g"] = (l.heads * l.vdim, d), (l.heads * l.vdim, d)
+            out[m + "a1"], out[m + "a2"], out[m + "a2.b"] = (l.rank, d), (l.heads * l.dim, l.rank), (l.heads * l.dim,)
+            out[m + "norm"] = (l.vdim,)
+            out[m + "o"] = (d, l.heads * l.vdim)
+        if l.ff:
+            out[p + "mlp.up"], out[p + "mlp.down"] = (l.ff, d), (d, l.ff)
+    out["final.norm"] = ()
+    out["head"] = (cfg.vocab_size, d)
+    return out
+
+
+@dataclass
+class StepLayout:
+    """All sequences of a step, prompt portions first, single decoded tokens behind them
+    (device tensors, int32)."""
+
+    cu_q: torch.Tensor                      # [B+1] row ranges
+    row_seq: torch.Tensor                   # [T] sequence of each row (< 0: padding row)
+    block_tables: torch.Tensor              # [B, max_blocks]
+    state_slots: Optional[torch.Tensor]     # [B] (< 0: padding row), None for models without state
+
+
+class HybridCache:
+    """Paged keys / values of the attention layers that own any, and the fp32 state slots of the
+    recurrent layers, in ONE pool. Key planes are [blocks, G, BS, dim], value planes
+    [blocks, G, BS, vdim] in the model's activation type; a state plane is [slots, size] fp32."""
+
+    def __init__(self, cfg: HybridConfig, num_blocks: int, block_size: int, num_slots: int, device,
+                 dtype: torch.dtype, alloc=None):
+        self.cfg, self.num_blocks, self.block_size, self.num_slots = cfg, num_blocks, block_size, num_slots
+        es = 4 if dtype == torch.float32 else 2
+        plan, off = [], 0
+
+        def take(nbytes: int) -> int:
+            nonlocal off
+            at = off
+            off = (off + nbytes + 255) // 256 * 256
+            return at
+        for i, l in enumerate(cfg.layers):
+            if l.owns_kv:
+                plan.append(("k", i, take(num_blocks * l.kv_heads * block_size * l.dim * es)))
+                plan.append(("v", i, take(num_blocks * l.kv_heads * block_size * l.vdim * es)))
+            elif l.state_size():
+                plan.append(("s", i, take(max(1, num_slots) * l.state_size() * 4)))
+        total = max(off, 256)
+        if alloc is None:
+            self.pool = torch.zeros(total // 2, dtype=torch.bfloat16, device=device)
+        else:
+            self.pool = alloc(total // 2)
+            ops.zero_(self.pool)
+        raw = self.pool.view(torch.uint8)
+        self._k: Dict[int, torch.Tensor] = {}
+        self._v: Dict[int, torch.Tensor] = {}
+        self._s: Dict[int, torch.Tensor] = {}
+        for kind, i, at in plan:
+            l = cfg.layers[i]
+            if kind == "k":
+                n = num_blocks * l.kv_heads * block_size * l.dim * es
+                self._k[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.dim)
+            elif kind == "v":
+                n = num_blocks * l.kv_heads * block_size * l.vdim * es
+                self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.vdim)
+            else:
+                n = max(1, num_slots) * l.state_size() * 4
+                self._s[i] = raw[at:at + n].view(torch.float32).view(max(1, num_slots), l.state_size())
+
+    def k(self, layer: int) -> torch.Tensor:
+        return self._k[layer]
+
+    def v(self, layer: int) -> torch.Tensor:
+        return self._v[layer]
+
+    def state(self, layer: int) -> torch.Tensor:
+        return self._s[layer]
+
+    def copy_blocks(self, src: torch.Tensor, dst: torch.Tensor) -> None:
+        # sequences with a state slot are never forked (csrc/core/kv_manager.cpp), so no block is
+        # ever shared and copied on write
+        raise NotImplementedError("hybrid decoders serve one chain per request: no copy-on-write")
+
+    @staticmethod
+    def bytes_per_block(cfg: HybridConfig, block_size: int, dtype: torch.dtype) -> int:
+        return max(1, cfg.kv_elems_per_token() * block_size * (4 if dtype == torch.float32 else 2))
+
+
+@dataclass
+class HybridLayer:
+    spec: LayerSpec
+    norm1: torch.Tensor                             # fp32 [1]
+    proj: ops.LinearWeight                          # fused input projections of the mixer
+    out: ops.LinearWeight
+    norm2: Optional[torch.Tensor] = None
+    up: Optional[ops.LinearWeight] = None
+    down: Optional[ops.LinearWeight] = None
+    q_norm: Optional[torch.Tensor] = None           # fp32 [H*D]
+    k_norm: Optional[torch.Tensor] = None
+    inv_freq: Optional[torch.Tensor] = None         # fp32 [rot_dims/2]
+    decay_up: Optional[ops.LinearWeight] = None     # gla: bottleneck -> decay logits
+    head_norm: Optional[torch.Tensor] = None        # gla: fp32 [vdim]
+
+
+class HybridModel:
+    """One Nidozen model on one device. Same surface as ``TransformerModel`` towards the engine:
+    ``forward`` (the residual stream of the step's rows), ``logits``, ``make_cache``."""
+
+    tp_rank, tp_size, ep_size, comm = 0, 1, 1, None
+    supports_embed = False          # pooled embeddings read bf16 final-normed rows; this stream is fp32
+    wants_layout = True
+
+    def __init__(self, cfg: HybridConfig, device, dtype: torch.dtype = torch.bfloat16) -> None:
+        cfg.validate()
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"{cfg.name}: activation type {dtype}: bf16 or fp32")
+        self.cfg, self.device, self.dtype = cfg, torch.device(device), dtype
+        self.hq, self.hkv = cfg.num_heads, cfg.num_kv_heads
+        self.embed: Optional[torch.Tensor] = None
+        self.final_norm: Optional[torch.Tensor] = None
+        self.lm_head: Optional[ops.LinearWeight] = None
+        self.layers: List[HybridLayer] = []
+        self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+
+    # ------------------------------------------------------------------ construction
+    def set_weights(self, get) -> None:
+        """``get(name) -> tensor`` with the checkpoint's names. Shapes are checked against the
+        configuration, by name, before anything is fused or packed."""
+        c, dev, dt = self.cfg, self.device, self.dtype
+        shapes = param_shapes(c)
+
+        def load(name: str) -> torch.Tensor:
+            t = get(name)
+            t = t.to(torch.float32) if hasattr(t, "to") else torch.as_tensor(t, dtype=torch.float32)
+            if tuple(t.shape) != tuple(shapes[name]):
+                raise ValueError(f"{c.name}: tensor {name!r} has shape {tuple(t.shape)}, the configuration implies "
+                                 f"{tuple(shapes[name])}")
+            return t.to(dev)
+
+        def lin(W: torch.Tensor, b: Optional[torch.Tensor] = None) -> ops.LinearWeight:
+            return ops.LinearWeight.from_dense(W, b, dev, dtype=dt, any_shape=True)
+
+        def f32(t: torch.Tensor) -> torch.Tensor:
+            return t.to(torch.float32).reshape(-1).contiguous()
+        self.embed = load("embed").to(dt).contiguous()
+        self.final_norm = f32(load("final.norm"))
+        self.lm_head = lin(load("head"))
+        self.layers = []
+        for i, l in enumerate(c.layers):
+            p, m = f"l{i}.", f"l{i}.mix."
+            kw = {}
+            if l.type == "attention":
+                Ws, bs = [load(m + "q")], [load(m + "q.b")]
+                if l.owns_kv:
+                    Ws += [load(m + "k"), load(m + "v")]
+                    bs += [load(m + "k.b"), load(m + "v.b")]
+                    kw["k_norm"] = f32(load(m + "k.norm"))
+                kw["q_norm"] = f32(load(m + "q.norm"))
+                half = l.rot_dims // 2
+                inv = torch.tensor([l.rot_base ** (-2.0 * j / l.rot_dims) for j in range(half)] or [0.0],
+                                   dtype=torch.float64)
+                kw["inv_freq"] = inv.to(torch.float32).to(dev)
+                proj, out = lin(torch.cat(Ws, 0), torch.cat(bs, 0)), lin(load(m + "o"), load(m + "o.b"))
+            elif l.type == "mingru":
+                bias = torch.cat([load(m + "z.b"), load(m + "x.b"), torch.zeros(l.width, device=dev)])
+                proj = lin(torch.cat([load(m + "z"), load(m + "x"), load(m + "g")], 0), bias)
+                out = lin(load(m + "o"))
+            else:
+                proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "a1")], 0))
+                kw["decay_up"] = lin(load(m + "a2"), load(m + "a2.b"))
+                kw["head_norm"] = f32(load(m + "norm"))
+                out = lin(load(m + "o"))
+            if l.ff:
+                kw.update(norm2=f32(load(p + "norm2")), up=lin(load(p + "mlp.up")), down=lin(load(p + "mlp.down")))
+            self.layers.append(HybridLayer(l, f32(load(p + "norm1")), proj, out, **kw))
+
+    @classmethod
+    def random_init(cls, cfg: HybridConfig, device, seed: int = 0, dtype: torch.dtype = torch.bfloat16,
+                    **_ignored) -> "HybridModel":
+        """Random weights of the configured shapes (benchmarks, smoke tests): N(0, 1/fan_in)
+        matrices, small biases, gains near one, decay biases that keep the states alive."""
+        m = cls(cfg, device, dtype)
+        shapes = param_shapes(cfg)
+        gen = torch.Generator()
+
+        def get(name: str) -> torch.Tensor:
+            shape = shapes[name]
+            gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFFFFFFFFFF)
+            if len(shape) == 2:
+                t = torch.randn(shape, generator=gen) * (1.0 if name == "embed" else shape[1] ** -0.5)
+            elif name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
+                t = 1.0 + 0.1 * torch.randn(shape, generator=gen)
+            elif name.endswith("a2.b"):
+                t = 2.0 + torch.randn(shape, generator=gen)
+            else:
+                t = 0.1 * torch.randn(shape, generator=gen)
+            return t.to(torch.bfloat16)
+        m.set_weights(get)
+        return m
+
+    def weight_bytes(self) -> int:
+        n = self.embed.numel() * self.embed.element_size() + self.lm_head.nbytes()
+        for L in self.layers:
+            for w in (L.proj, L.out, L.up, L.down, L.decay_up):
+                n += w.nbytes() if w is not None else 0
+        return n
+
+    # ------------------------------------------------------------------ engine surface
+    def make_cache(self, num_blocks: int, block_size: int, num_slots: int, alloc=None) -> HybridCache:
+        return HybridCache(self.cfg, num_blocks, block_size, num_slots, self.device, self.dtype, alloc)
+
+    def cache_bytes_per_block(self, block_size: int) -> int:
+        return HybridCache.bytes_per_block(self.cfg, block_size, self.dtype)
+
+    def state_slots_needed(self, max_seqs: int) -> int:
+        return max_seqs if self.cfg.has_state else 0
+
+    def decode_capturable(self, rows: int) -> bool:
+        return True
+
+    def _decode_layout(self, meta, B: int) -> StepLayout:
+        """A pure decode step described the old way (one row per sequence): rows are sequences."""
+        e = self._rows.get(B)
+        if e is None:
+            e = (torch.arange(B + 1, dtype=torch.int32, device=self.device),
+                 torch.arange(B, dtype=torch.int32, device=self.device))
+            self._rows[B] = e
+        return StepLayout(e[0], e[1], meta.block_tables, None)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, token_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, meta,
+                cache: HybridCache, taps: Optional[list] = None) -> torch.Tensor:
+        """The fp32 residual stream [T, d] after the last layer for the step's rows (``logits``
+        applies the final norm). ``taps`` (a list) receives a copy of the stream after every layer."""
+        c, dt, eps = self.cfg, self.dtype, self.cfg.rms_eps
+        lay: StepLayout = getattr(meta, "layout", None) or self._decode_layout(meta, token_ids.numel())
+        if c.has_state and lay.state_slots is None:
+            raise ValueError(f"{c.name}: the step names no state slots (the engine's KV manager must be made with slots)")
+        x, xa = ops.embed_rows(token_ids, self.embed, dt, meta.token_feed)
+        for i, L in enumerate(self.layers):
+            l = L.spec
+            if l.type == "attention":
+                y = self._attention(i, L, xa, positions, slot_mapping, lay, cache)
+            elif l.type == "mingru":
+                zxg = ops.linear(xa, L.proj, out_f32=True)
+                y = ops.mingru_scan(zxg, cache.state(i), lay.cu_q, positions, lay.state_slots, dt)
+                y = ops.linear(y, L.out, out_f32=True)
+            else:
+                y = self._gla(i, L, xa, positions, lay, cache)
+            xa = ops.scalar_norm_add(x, y, L.norm1, eps, dt)
+            if L.up is not None:
+                if L.up.is_packed or not x.is_cuda:
+                    u = ops.relu2(ops.linear(xa, L.up, out_f32=True), dt)
+                else:
+                    u = ops.linear_any(xa, L.up, out_f32=dt == torch.float32, epi_relu2=True)
+                xa = ops.scalar_norm_add(x, ops.linear(u, L.down, out_f32=True), L.norm2, eps, dt)
+            if taps is not None:
+                taps.append(x.clone())
+        return x
+
+    def _attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
+        l = L.spec
+        src = i if l.owns_kv else l.kv_from
+        kc, vc = cache.k(src), cache.v(src)
+        qkv = ops.linear(xa, L.proj, out_f32=True)
+        q = ops.qkv_prep(qkv, L.q_norm, L.k_norm, L.inv_freq, positions, slot_mapping, kc if l.owns_kv else None,
+                         vc if l.owns_kv else None, l.heads, l.kv_heads, l.dim, l.vdim, l.rot_dims, l.rot_base,
+                         self.cfg.rms_eps)
+        a = ops.attn_masked(q, kc, vc, lay.block_tables, lay.cu_q, lay.row_seq, positions, l.heads, l.kv_heads, l.dim,
+                            l.vdim, l.scale, l.chunk, l.window, self.dtype)
+        return ops.linear(a, L.out, out_f32=True)
+
+    def _gla(self, i: int, L: HybridLayer, xa, positions, lay: StepLayout, cache: HybridCache):
+        l = L.spec
+        hd, hv = l.heads * l.dim, l.heads * l.vdim
+        proj = ops.linear(xa, L.proj, out_f32=True)                 # q | k | v | gate | bottleneck
+        logits = ops.linear_any(proj[:, 2 * hd + 2 * hv:].contiguous(), L.decay_up) if not L.decay_up.is_packed \
+            else ops.linear(proj[:, 2 * hd + 2 * hv:].to(torch.bfloat16).contiguous(), L.decay_up, out_f32=True)
+        o = ops.gla_scan(proj, logits, cache.state(i), lay.cu_q, positions, lay.state_slots, l.heads, l.dim, l.vdim,
+                         l.tau)
+        y = ops.headnorm_gate(o, L.head_norm, proj[:, 2 * hd + hv:2 * hd + 2 * hv], l.vdim, self.cfg.rms_eps, self.dtype)
+        return ops.linear(y, L.out, out_f32=True)
+
+    def logits(self, hidden_rows: torch.Tensor) -> torch.Tensor:
+        """fp32 logits [R, V] of the given rows of the residual stream (final norm, then the head)."""
+        xa = ops.scalar_norm_add(hidden_rows, None, self.final_norm, self.cfg.rms_eps, self.dtype)
+        return ops.linear(xa, self.lm_head, out_f32=True)
+
+    def target_logprobs(self, hidden_rows: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        return ops.logprob_gather(self.logits(hidden_rows), ids)

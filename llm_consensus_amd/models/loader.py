@@ -132,7 +132,34 @@ class SafetensorsIndex:
 
 
 def load_model(path: str, device, tp_rank: int = 0, tp_size: int = 1, comm=None,
-               cfg: Optional[ModelConfig] = None, ep_size: int = 1, ep_mode: str = "allreduce") -> TransformerModel:
+               cfg: Optional[ModelConfig] = None, ep_size: int = 1, ep_mode: str = "allreduce", dtype=None):
+    """Loads a checkpoint directory with the model class its ``config.json`` names
+    (models/registry.py). ``dtype`` (bf16 | fp32) is for families that serve both."""
+    from .registry import resolve
+
+    fam = resolve(path)
+    if fam.name == "transformer":
+        if dtype not in (None, torch.bfloat16):
+            raise ValueError("the transformer families are served in bf16 only")
+        return load_transformer(path, device, tp_rank, tp_size, comm, cfg, ep_size, ep_mode)
+    if tp_size > 1 or ep_size > 1:
+        raise ValueError(f"{path}: the {fam.name} family runs on one device")
+    return fam.load(path, device, dtype=dtype or torch.bfloat16)
+
+
+def load_hybrid(path: str, device, dtype=torch.bfloat16):
+    """A hybrid decoder's checkpoint: ``config.json`` + ``model.safetensors`` (bf16 tensors)."""
+    from .hybrid import HybridModel, config_from_path
+
+    model = HybridModel(config_from_path(path), device, dtype)
+    index = SafetensorsIndex(path, None)
+    model.set_weights(lambda name: index.get(name).materialize())
+    return model
+
+
+def load_transformer(path: str, device, tp_rank: int = 0, tp_size: int = 1, comm=None,
+                     cfg: Optional[ModelConfig] = None, ep_size: int = 1,
+                     ep_mode: str = "allreduce") -> TransformerModel:
     cfg = cfg or from_hf_config(path)
     model = TransformerModel(cfg, device, tp_rank, tp_size, comm, ep_size, ep_mode)
     index = SafetensorsIndex(path, PinnedStager(model.device))
@@ -187,9 +214,10 @@ def build_model(spec, device, tp_rank: int = 0, tp_size: int = 1, comm=None, ep_
     dev = torch.device(device)
     if dev.type == "cuda":
         from .. import runtime
-        from .config import from_hf_config
+        from .registry import resolve
 
-        mc = from_hf_config(spec.path) if getattr(spec, "path", None) else get_preset(spec.preset or "tiny-llama")
+        mc = resolve(spec.path).read_config(spec.path) if getattr(spec, "path", None) \
+            else get_preset(spec.preset or "tiny-llama")
         with torch.cuda.device(dev):
             runtime.require_hbm(mc.weight_bytes() // max(1, tp_size, ep_size), f"model {getattr(spec, 'name', '?')}")
     if getattr(spec, "path", None):

@@ -44,6 +44,10 @@ class AttnMeta:
     prefill_tokens: int = 0
     # Decode steps launched ahead of the previous step's results: (tokens, rows), see ops.embed.
     token_feed: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+    # All sequences of the step in one description (row ranges, row -> sequence, block tables,
+    # state slots), for models whose mixers treat prompt portions and decoded tokens alike
+    # (models/hybrid.py: StepLayout). The engine fills it for models that ask (``wants_layout``).
+    layout: Optional[object] = None
 
 
 @dataclass
@@ -185,6 +189,20 @@ class TransformerModel:
                 lw.gate_up = ops.LinearWeight.from_dense(gu, None, dev, swiglu=True)
                 lw.down = ops.LinearWeight.from_dense(bf(get(p + "mlp.down_proj.weight")[:, sl]).contiguous(), None, dev)
             self.layers.append(lw)
+
+    # ---- what the engine asks a model about its cache (models/hybrid.py answers differently) ----
+    wants_layout = False
+    supports_embed = True
+
+    def make_cache(self, num_blocks: int, block_size: int, num_slots: int = 0, alloc=None) -> KVCache:
+        return KVCache(self.cfg, num_blocks, block_size, self.device, self.hkv, alloc=alloc)
+
+    def cache_bytes_per_block(self, block_size: int) -> int:
+        return KVCache.bytes_per_block(self.cfg, block_size, self.hkv)
+
+    def state_slots_needed(self, max_seqs: int) -> int:
+        """Per-sequence state slots the KV manager must hand out (none: attention only)."""
+        return 0
 
     def decode_capturable(self, rows: int) -> bool:
         """Whether a decode step of ``rows`` sequences can be recorded into a hipGraph: every

@@ -119,13 +119,20 @@ class LinearWeight:
         return self.data.dim() == 4
 
     @classmethod
-    def from_dense(cls, W: torch.Tensor, bias: Optional[torch.Tensor] = None, device=None, swiglu: bool = False):
-        """W row-major [N, K] in final row order (already interleaved when swiglu)."""
+    def from_dense(cls, W: torch.Tensor, bias: Optional[torch.Tensor] = None, device=None, swiglu: bool = False,
+                   dtype: torch.dtype = torch.bfloat16, any_shape: bool = False):
+        """W row-major [N, K] in final row order (already interleaved when swiglu). With
+        ``any_shape`` a weight the MFMA kernels do not take (fp32, or a reduction depth that is
+        no multiple of 64) stays row-major on the GPU too and goes through the shape-agnostic
+        kernel (hybrid.hip); without it such a weight is an error at the first product."""
         device = torch.device(device) if device is not None else W.device
         N, K = W.shape
-        W = W.to(device=device, dtype=torch.bfloat16)
-        b = bias.to(device=device, dtype=torch.bfloat16).contiguous() if bias is not None else None
-        data = pack_weight(W) if device.type == "cuda" else W.contiguous()
+        W = W.to(device=device, dtype=dtype)
+        b = bias.to(device=device, dtype=dtype).contiguous() if bias is not None else None
+        plain = any_shape and (dtype != torch.bfloat16 or K % 64 != 0)
+        if plain and swiglu:
+            raise ValueError("the shape-agnostic product has no SwiGLU epilogue")
+        data = pack_weight(W) if (device.type == "cuda" and not plain) else W.contiguous()
         return cls(data, N, K, b, swiglu)
 
     def dense(self) -> torch.Tensor:
@@ -235,7 +242,11 @@ def linear(x: torch.Tensor, w: LinearWeight, out_f32: bool = False, defer_reduce
         return y if out_f32 else y.to(x.dtype)
     h = _hip()
     if not w.is_packed:
-        raise RuntimeError("GPU linear needs packed weights (LinearWeight.from_dense on a cuda device)")
+        if w.swiglu or w.data.dim() != 2:
+            raise RuntimeError("GPU linear needs packed weights (LinearWeight.from_dense on a cuda device)")
+        return linear_any(x, w, out_f32)
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"the MFMA products take bf16 activations, got {x.dtype}")
     x = x.contiguous()
     epi = EPI_SWIGLU if w.swiglu else (EPI_F32 if out_f32 else EPI_BF16)
     y = torch.empty(M, out_n, dtype=torch.float32 if (out_f32 and not w.swiglu) else torch.bfloat16, device=x.device)
@@ -627,6 +638,8 @@ def gather_rows(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
     gather is what it is)."""
     if not x.is_cuda:
         return x[rows.long()]
+    if x.dtype == torch.float32:           # the fp32 residual stream of the hybrid decoders
+        return embed_rows(rows, x.contiguous(), None)[0]
     return embed(rows, x)
 
 
@@ -851,3 +864,186 @@ def moe_ffn(x: torch.Tensor, Wr: torch.Tensor, w_gate_up: ExpertWeights, w_down:
     the result is this rank's partial sum."""
     ids, wts = moe_route(x, Wr, topk)
     return moe_experts(x, ids, wts, w_gate_up, w_down, expert_lo, Wr.shape[0])
+
+
+# ---------------------------------------------------------------------------- hybrid decoders
+# Ops of hybrid decoder designs (csrc/kernels/hybrid.hip): an fp32 residual stream with scalar-gain
+# norms on the sublayer outputs, recurrences over per-sequence state slots, attention with separate
+# key / value widths under a chunk or window mask. ``act_dtype`` (bf16 or fp32) is the type of what
+# feeds the next matrix product; everything else is fp32. CPU tensors go to ops.reference.
+def _f32flag(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return 1
+    if dtype == torch.bfloat16:
+        return 0
+    raise TypeError(f"activation type {dtype}: bf16 or fp32")
+
+
+def linear_any(x: torch.Tensor, w: LinearWeight, out_f32: bool = True, epi_relu2: bool = False) -> torch.Tensor:
+    """y = x W^T (+ bias) for a row-major weight of any shape and type (fp32 accumulation on the
+    vector ALUs). ``epi_relu2``: the square of relu in the epilogue."""
+    M = x.shape[0]
+    odt = torch.float32 if out_f32 else torch.bfloat16
+    if x.shape[1] != w.k:
+        raise ValueError(f"linear_any: activations of width {x.shape[1]} against a weight of depth {w.k}")
+    if not x.is_cuda:
+        y = ref.linear(x, w.dense(), w.bias, torch.float32)
+        return (torch.relu(y).pow(2) if epi_relu2 else y).to(odt)
+    if w.is_packed:
+        raise ValueError("linear_any takes row-major weights")
+    x = x.contiguous()
+    y = torch.empty(M, w.n, dtype=odt, device=x.device)
+    _hip().call("lc_gemm_any", x.data_ptr(), _f32flag(x.dtype), w.data.data_ptr(), _f32flag(w.data.dtype),
+                _hip().ptr(w.bias), y.data_ptr(), 1 if out_f32 else 0, M, w.n, w.k, 1 if epi_relu2 else 0)
+    return y
+
+
+def embed_rows(ids: torch.Tensor, E: torch.Tensor, act_dtype: Optional[torch.dtype],
+               feed: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+    """Rows E[ids] as (fp32 [T, d], copy in ``act_dtype`` or None). E is bf16 or fp32; with
+    ``act_dtype`` fp32 the copy IS the fp32 tensor. ``feed`` as in ``embed``. Also the row gather
+    of an fp32 matrix."""
+    T, d = ids.numel(), E.shape[1]
+    if not ids.is_cuda:
+        if feed is not None:
+            tok, rows = feed
+            ids = torch.where(rows >= 0, tok[rows.clamp_min(0).long()].to(ids.dtype), ids)
+        x = ref.embed(ids, E).float()
+        return x, (x if act_dtype in (None, torch.float32) else x.to(act_dtype))
+    x = torch.empty(T, d, dtype=torch.float32, device=E.device)
+    xa = torch.empty(T, d, dtype=act_dtype, device=E.device) if act_dtype == torch.bfloat16 else None
+    _hip().call("lc_embed_rows", ids.data_ptr(), E.data_ptr(), _f32flag(E.dtype), x.data_ptr(), _hip().ptr(xa), 0, T, d,
+                E.shape[0], feed[0].data_ptr() if feed is not None else None,
+                feed[1].data_ptr() if feed is not None else None)
+    return x, (xa if xa is not None else (x if act_dtype is not None else None))
+
+
+def scalar_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
+                    act_dtype: torch.dtype) -> torch.Tensor:
+    """x (fp32 residual stream, in place) += y / sqrt(mean(y^2) + eps) * gain and the new x in
+    ``act_dtype``; without ``y``: the normed x in ``act_dtype`` (x untouched). ``gain`` is an
+    fp32 tensor of one element."""
+    if not x.is_cuda:
+        return ref.scalar_norm_add(x, y, gain, eps, act_dtype)
+    T, d = x.shape
+    if y is not None and (y.shape != x.shape or y.dtype != torch.float32):
+        raise ValueError("scalar_norm_add: the sublayer output must be fp32 of the stream's shape")
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("scalar_norm_add: the residual stream is a contiguous fp32 tensor")
+    alias = y is not None and act_dtype == torch.float32       # the fp32 'copy' is the stream itself
+    xa = None if alias else torch.empty(T, d, dtype=act_dtype, device=x.device)
+    _hip().call("lc_scalar_norm_add", x.data_ptr(), _hip().ptr(y.contiguous() if y is not None else None),
+                gain.data_ptr(), float(eps), _hip().ptr(xa), _f32flag(act_dtype), T, d)
+    return x if alias else xa
+
+
+def relu2(y: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+    if not y.is_cuda:
+        return ref.relu2(y, act_dtype)
+    y = y.contiguous()
+    out = torch.empty(y.shape, dtype=act_dtype, device=y.device)
+    _hip().call("lc_relu2", y.data_ptr(), out.data_ptr(), _f32flag(act_dtype), y.numel())
+    return out
+
+
+def mingru_scan(zxg: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
+                slots: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+    """minGRU over the step's sequences: zxg fp32 [T, 3w] (update-gate logits | candidate
+    pre-activations | output-gate logits), state fp32 [slots, w] (updated in place). Returns
+    S * silu(g) [T, w] in ``act_dtype``."""
+    if not zxg.is_cuda:
+        return ref.mingru_scan(zxg, state, cu_q, positions, slots, act_dtype)
+    T, w = zxg.shape[0], zxg.shape[1] // 3
+    if zxg.dtype != torch.float32 or state.dtype != torch.float32 or state.shape[1] != w:
+        raise ValueError("mingru_scan: fp32 projections [T, 3w] and fp32 state [slots, w]")
+    zxg = zxg.contiguous()
+    out = torch.empty(T, w, dtype=act_dtype, device=zxg.device)
+    _hip().call("lc_mingru_scan", zxg.data_ptr(), state.data_ptr(), cu_q.data_ptr(), positions.data_ptr(),
+                slots.data_ptr(), out.data_ptr(), _f32flag(act_dtype), slots.numel(), w)
+    return out
+
+
+def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+             positions: torch.Tensor, slots: torch.Tensor, H: int, D: int, Dv: int, tau: float) -> torch.Tensor:
+    """Gated linear attention over the step's sequences. proj fp32 [T, >= 2HD + HDv] holds
+    q | k | v in its first columns, decay_logits fp32 [T, HD]; state fp32 [slots, H*D*Dv]
+    (updated in place). Returns the un-normed read-out fp32 [T, H*Dv]."""
+    if not proj.is_cuda:
+        return ref.gla_scan(proj, decay_logits, state, cu_q, positions, slots, H, D, Dv, tau)
+    T = proj.shape[0]
+    if proj.dtype != torch.float32 or decay_logits.dtype != torch.float32 or state.dtype != torch.float32:
+        raise ValueError("gla_scan: fp32 inputs and state")
+    if state.shape[1] != H * D * Dv or decay_logits.shape[1] != H * D or proj.stride(1) != 1:
+        raise ValueError("gla_scan: shapes do not fit the head sizes")
+    decay_logits = decay_logits.contiguous()
+    out = torch.empty(T, H * Dv, dtype=torch.float32, device=proj.device)
+    _hip().call("lc_gla_scan", proj.data_ptr(), proj.stride(0), decay_logits.data_ptr(), state.data_ptr(),
+                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), slots.numel(), H, D, Dv,
+                float(tau))
+    return out
+
+
+def headnorm_gate(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, Dv: int, eps: float,
+                  act_dtype: torch.dtype) -> torch.Tensor:
+    """Per head of width Dv: o / sqrt(mean(o^2) + eps) * w, times silu(gate). ``gate`` may be a
+    column slice of a wider fp32 matrix."""
+    if not o.is_cuda:
+        return ref.headnorm_gate(o, w, gate, Dv, eps, act_dtype)
+    T, n = o.shape
+    if gate.shape != o.shape or gate.stride(1) != 1 or o.dtype != torch.float32 or gate.dtype != torch.float32:
+        raise ValueError("headnorm_gate: fp32 read-out and gate of one shape")
+    o = o.contiguous()
+    out = torch.empty(T, n, dtype=act_dtype, device=o.device)
+    _hip().call("lc_headnorm_gate", o.data_ptr(), w.data_ptr(), gate.data_ptr(), gate.stride(0), out.data_ptr(),
+                _f32flag(act_dtype), T, n // Dv, Dv, float(eps))
+    return out
+
+
+def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Tensor], inv_freq: torch.Tensor,
+             positions: torch.Tensor, slot_mapping: torch.Tensor, k_cache: Optional[torch.Tensor],
+             v_cache: Optional[torch.Tensor], H: int, G: int, D: int, Dv: int, rot_dims: int, rot_base: float,
+             eps: float) -> torch.Tensor:
+    """Attention pre-processing in one launch: RMS norm of the whole query (and key) projection
+    with per-coordinate weights, partial rotate-half rotary positions, unit-RMS value heads, and
+    the write of keys [blocks, G, BS, D] / values [blocks, G, BS, Dv] at the rows' slots. A layer
+    that reads another layer's keys passes no caches. Returns q fp32 [T, H*D]."""
+    if not qkv.is_cuda:
+        return ref.qkv_prep(qkv, q_norm, k_norm, positions, slot_mapping, k_cache, v_cache, H, G, D, Dv, rot_dims,
+                            rot_base, eps)
+    T = qkv.shape[0]
+    if qkv.dtype != torch.float32 or qkv.stride(1) != 1:
+        raise ValueError("qkv_prep: fp32 projections")
+    has_kv = k_cache is not None
+    if has_kv and (k_cache.dtype != v_cache.dtype or k_cache.shape[1:] != (G, k_cache.shape[2], D)
+                   or v_cache.shape[1:] != (G, k_cache.shape[2], Dv)):
+        raise ValueError("qkv_prep: cache planes do not fit the head sizes")
+    q = torch.empty(T, H * D, dtype=torch.float32, device=qkv.device)
+    _hip().call("lc_qkv_prep", qkv.data_ptr(), qkv.stride(0), q_norm.data_ptr(), _hip().ptr(k_norm), inv_freq.data_ptr(),
+                positions.data_ptr(), slot_mapping.data_ptr(), _hip().ptr(k_cache), _hip().ptr(v_cache),
+                _f32flag(k_cache.dtype) if has_kv else 0, q.data_ptr(), T, H, G, D, Dv,
+                k_cache.shape[2] if has_kv else 1, rot_dims, float(eps), 1 if has_kv else 0)
+    return q
+
+
+def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                cu_q: torch.Tensor, row_seq: torch.Tensor, positions: torch.Tensor, H: int, G: int, D: int, Dv: int,
+                scale: float, chunk: int, window: int, act_dtype: torch.dtype) -> torch.Tensor:
+    """Attention of fp32 queries [T, H*D] over paged keys / values of widths D / Dv. The row at
+    position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
+    j > p - window (``window`` > 0), counted from the start of its sequence. ``row_seq`` [T]
+    names each row's sequence (row of ``block_tables``). Serves portions of prompts and single
+    decoded tokens alike; scores, weights and sums are fp32."""
+    if not q.is_cuda:
+        return ref.attn_masked(q, k_cache, v_cache, block_tables, cu_q, positions, H, G, D, Dv, scale, chunk, window,
+                               act_dtype)
+    T = q.shape[0]
+    if q.dtype != torch.float32 or not q.is_contiguous() or k_cache.dtype != v_cache.dtype:
+        raise ValueError("attn_masked: contiguous fp32 queries, caches of one type")
+    if k_cache.shape[1:] != (G, k_cache.shape[2], D) or v_cache.shape[1:] != (G, k_cache.shape[2], Dv):
+        raise ValueError("attn_masked: cache planes do not fit the head sizes")
+    out = torch.empty(T, H * Dv, dtype=act_dtype, device=q.device)
+    _hip().call("lc_attn_masked", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _f32flag(k_cache.dtype),
+                block_tables.data_ptr(), block_tables.shape[1], row_seq.data_ptr(), positions.data_ptr(),
+                out.data_ptr(), _f32flag(act_dtype), T, H, G, D, Dv, k_cache.shape[2], float(scale), int(chunk),
+                int(window))
+    return out

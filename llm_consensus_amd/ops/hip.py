@@ -57,6 +57,16 @@ _SIGNATURES = {
     "lc_ep_pack": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "lc_ep_recv_index": [_P, _I, _I, _I, _P, _P, _P],
     "lc_scatter_rows": [_P, _P, _P, _I, _I, _P, _P],
+    # hybrid decoders (hybrid.hip)
+    "lc_embed_rows": [_P, _P, _I, _P, _P, _I, _I, _I, _I, _P, _P, _P],
+    "lc_scalar_norm_add": [_P, _P, _P, _F, _P, _I, _I, _I, _P],
+    "lc_relu2": [_P, _P, _I, _L, _P],
+    "lc_mingru_scan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "lc_gla_scan": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P],
+    "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
+    "lc_qkv_prep": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "lc_gemm_any": [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
 }
 
 _lib = None
@@ -71,7 +81,11 @@ def lib() -> ctypes.CDLL:
     if _lib is None:
         l = kernels()
         for name, argtypes in _SIGNATURES.items():
-            fn = getattr(l, name)
+            # a library built for some model families only (build_native.py: source groups)
+            # lacks the launchers of the others; calling one of those raises AttributeError
+            fn = getattr(l, name, None)
+            if fn is None:
+                continue
             fn.argtypes = argtypes
             fn.restype = c_int
         _lib = l

@@ -281,3 +281,152 @@ def embed_pool(hidden: torch.Tensor, cu: torch.Tensor, mode: int = 0) -> torch.T
         n = v.norm()
         outs.append(v / n if n > 0 else v)
     return torch.stack(outs).to(hidden.device)
+
+
+# ------------------------------------------------------------------ hybrid decoders: fp32 residual stream
+# Mixers of hybrid decoder designs (scalar-gain output norms on an fp32 residual stream, gated
+# recurrences with per-sequence state slots, attention with separate key / value widths under a
+# chunk or window mask). Sequences of a step are described by ``cu_q`` [B+1] (row ranges),
+# ``positions`` [T] and ``slots`` [B] (state slot per sequence, < 0 = skip the sequence).
+def scalar_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], gain: torch.Tensor, eps: float, act_dtype):
+    """x (fp32, in place) += y / sqrt(mean(y^2) + eps) * gain; without ``y`` the normed x itself is
+    returned instead and x stays. Returns the result in ``act_dtype``."""
+    if y is None:
+        v = x.float()
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * gain.float()).to(act_dtype)
+    v = y.float()
+    x.add_(v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * gain.float())
+    return x.to(act_dtype)
+
+
+def relu2(y: torch.Tensor, act_dtype) -> torch.Tensor:
+    return torch.relu(y.float()).pow(2).to(act_dtype)
+
+
+def mingru_scan(zxg: torch.Tensor, state: torch.Tensor, cu_q, positions, slots, act_dtype) -> torch.Tensor:
+    """zxg fp32 [T, 3w] = (update-gate logits, candidate pre-activations, output-gate logits).
+    S <- (1 - z) S + z c with z = sigmoid(.), c = u + 1/2 for u >= 0 and sigmoid(u) below;
+    returns S * silu(g) [T, w]. A sequence whose first row is at position 0 starts from zero."""
+    T, w = zxg.shape[0], zxg.shape[1] // 3
+    out = torch.zeros(T, w, dtype=torch.float32, device=zxg.device)
+    z = torch.sigmoid(zxg[:, :w].float())
+    u = zxg[:, w:2 * w].float()
+    c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = zxg[:, 2 * w:].float()
+    for b in range(len(slots)):
+        r0, r1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(slots[b])
+        if slot < 0 or r1 <= r0:
+            continue
+        S = torch.zeros(w, dtype=torch.float32, device=zxg.device) if int(positions[r0]) == 0 else state[slot].clone()
+        for t in range(r0, r1):
+            S = (1 - z[t]) * S + z[t] * c[t]
+            out[t] = S
+        state[slot] = S
+    return (out * g * torch.sigmoid(g)).to(act_dtype)
+
+
+def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor, cu_q, positions, slots,
+             H: int, D: int, Dv: int, tau: float) -> torch.Tensor:
+    """proj fp32 [T, >= 2HD + HDv]: columns (q | k | v); decay_logits fp32 [T, HD].
+    Per head S <- diag(a) S + k v^T with a = sigmoid(logit)^(1/tau), o = S^T (q / sqrt(D)).
+    state [slots, H*D*Dv] fp32. Returns o fp32 [T, H*Dv]."""
+    T = proj.shape[0]
+    q = proj[:, :H * D].float().view(T, H, D) * (D ** -0.5)
+    k = proj[:, H * D:2 * H * D].float().view(T, H, D)
+    v = proj[:, 2 * H * D:2 * H * D + H * Dv].float().view(T, H, Dv)
+    a = torch.exp(torch.nn.functional.logsigmoid(decay_logits.float()) / tau).view(T, H, D)
+    out = torch.zeros(T, H, Dv, dtype=torch.float32, device=proj.device)
+    for b in range(len(slots)):
+        r0, r1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(slots[b])
+        if slot < 0 or r1 <= r0:
+            continue
+        S = state[slot].view(H, D, Dv).clone()
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for t in range(r0, r1):
+            S = a[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S.reshape(-1)
+    return out.view(T, H * Dv)
+
+
+def headnorm_gate(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, Dv: int, eps: float, act_dtype) -> torch.Tensor:
+    """Per head of width Dv: o / sqrt(mean(o^2) + eps) * w, times silu(gate)."""
+    T = o.shape[0]
+    v = o.float().view(T, -1, Dv)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    g = gate.float()
+    return (v.view(T, -1) * g * torch.sigmoid(g)).to(act_dtype)
+
+
+def rope_partial(x: torch.Tensor, positions: torch.Tensor, dims: int, base: float) -> torch.Tensor:
+    """x fp32 [T, heads, D]: the first ``dims`` coordinates of each head rotate (coordinate i with
+    i + dims/2, angle position * base^(-2i/dims)), the rest pass."""
+    half = dims // 2
+    if half == 0:
+        return x
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -2.0 * torch.arange(half, dtype=torch.float64) / dims).float().to(x.device)
+    ang = positions.float()[:, None] * f[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
+
+
+def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Tensor], positions, slot_mapping,
+             k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], H: int, G: int, D: int, Dv: int,
+             rot_dims: int, rot_base: float, eps: float) -> torch.Tensor:
+    """qkv fp32 [T, H*D (+ G*D + G*Dv)]. Queries (and keys) are RMS-normed over their WHOLE
+    projection with a weight per coordinate, then rotated; each value head is scaled to unit RMS.
+    Keys go to k_cache [blocks, G, BS, D], values to v_cache [blocks, G, BS, Dv] at the rows'
+    slots (skipped when the layer has no keys of its own: ``k_cache`` None). Returns q fp32 [T, H*D]."""
+    T = qkv.shape[0]
+    q = qkv[:, :H * D].float()
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()
+    q = rope_partial(q.view(T, H, D), positions, rot_dims, rot_base).reshape(T, H * D)
+    if k_cache is not None:
+        k = qkv[:, H * D:(H + G) * D].float()
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.float()
+        k = rope_partial(k.view(T, G, D), positions, rot_dims, rot_base)
+        v = qkv[:, (H + G) * D:(H + G) * D + G * Dv].float().view(T, G, Dv)
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        BS = k_cache.shape[2]
+        slots = slot_mapping.long()
+        ok = slots >= 0
+        blk, off = slots[ok] // BS, slots[ok] % BS
+        k_cache[blk, :, off, :] = k[ok].to(k_cache.dtype)
+        v_cache[blk, :, off, :] = v[ok].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions, H: int, G: int, D: int, Dv: int,
+                scale: float, chunk: int, window: int, act_dtype) -> torch.Tensor:
+    """q fp32 [T, H*D]; paged keys [blocks, G, BS, D] and values [blocks, G, BS, Dv]. The row at
+    position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
+    j > p - window (``window`` > 0). Scores, softmax and the weighted sum in fp32."""
+    T = q.shape[0]
+    out = torch.zeros(T, H * Dv, dtype=torch.float32, device=q.device)
+    BS = k_cache.shape[2]
+    rep = H // G
+    for b in range(len(cu_q) - 1):
+        r0, r1 = int(cu_q[b]), int(cu_q[b + 1])
+        if r1 <= r0:
+            continue
+        pos = positions[r0:r1].long()
+        n = int(pos.max()) + 1
+        nb = (n + BS - 1) // BS
+        blocks = block_tables[b, :nb].long()
+        K = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :n].float()
+        V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, Dv)[:, :n].float()
+        Q = q[r0:r1].float().view(r1 - r0, G, rep, D)
+        sc = torch.einsum("qgrd,gkd->grqk", Q, K) * scale
+        key = torch.arange(n, device=q.device)[None, :]
+        mask = key <= pos[:, None]
+        if chunk > 0:
+            mask &= key >= (pos[:, None] // chunk) * chunk
+        if window > 0:
+            mask &= key > pos[:, None] - window
+        sc = sc.masked_fill(~mask[None, None], float("-inf"))
+        o = torch.einsum("grqk,gkv->qgrv", torch.softmax(sc, dim=-1), V)
+        out[r0:r1] = o.reshape(r1 - r0, H * Dv)
+    return out.to(act_dtype)

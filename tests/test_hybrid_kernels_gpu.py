@@ -1,0 +1,150 @@
+"""HIP kernels of the hybrid decoders (csrc/kernels/hybrid.hip) against the plain PyTorch fp32
+versions of the same ops (ops/reference.py), one op at a time, in both activation types and at
+sizes that are not multiples of anything convenient."""
+import pytest
+import torch
+
+from llm_consensus_amd import ops
+from llm_consensus_amd.ops import reference as ref
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ACTS = [torch.bfloat16, torch.float32]
+
+
+def _tol(dt):
+    return dict(atol=2e-2, rtol=2e-2) if dt == torch.bfloat16 else dict(atol=2e-5, rtol=2e-5)
+
+
+def _seqs(lens, starts):
+    """cu_q, positions, row_seq for sequences of the given lengths that start at the given positions."""
+    cu, pos, rs = [0], [], []
+    for b, (n, s) in enumerate(zip(lens, starts)):
+        cu.append(cu[-1] + n)
+        pos += list(range(s, s + n))
+        rs += [b] * n
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32)  # noqa: E731
+    return i32(cu), i32(pos), i32(rs)
+
+
+@pytest.mark.parametrize("a_dt,w_dt,out_f32", [(torch.bfloat16, torch.bfloat16, True), (torch.float32, torch.bfloat16, True),
+                                              (torch.float32, torch.float32, True), (torch.bfloat16, torch.bfloat16, False)])
+@pytest.mark.parametrize("M,N,K", [(1, 7, 16), (5, 130, 100), (131, 64, 320), (70, 333, 48)])
+def test_gemm_any(a_dt, w_dt, out_f32, M, N, K):
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    x = torch.randn(M, K, generator=g).to(a_dt)
+    W = (torch.randn(N, K, generator=g) / K ** 0.5).to(w_dt)
+    b = torch.randn(N, generator=g).to(w_dt)
+    for relu2 in (False, True):
+        w = ops.LinearWeight.from_dense(W, b, DEV, dtype=w_dt, any_shape=True)
+        if w.is_packed:
+            continue
+        y = ops.linear_any(x.to(DEV), w, out_f32=out_f32, epi_relu2=relu2).float().cpu()
+        want = x.float() @ W.float().T + b.float()
+        want = torch.relu(want) ** 2 if relu2 else want
+        tol = dict(atol=1e-4, rtol=1e-4) if out_f32 else dict(atol=3e-2, rtol=2e-2)
+        torch.testing.assert_close(y, want, **tol)
+
+
+@pytest.mark.parametrize("dt", ACTS)
+def test_embed_rows_and_scalar_norm(dt):
+    g = torch.Generator().manual_seed(1)
+    E = torch.randn(50, 72, generator=g).to(dt)
+    ids = torch.randint(0, 50, (9,), generator=g, dtype=torch.int32)
+    x, xa = ops.embed_rows(ids.to(DEV), E.to(DEV), dt)
+    torch.testing.assert_close(x.cpu(), E[ids.long()].float())
+    torch.testing.assert_close(xa.float().cpu(), E[ids.long()].float())
+    y = torch.randn(9, 72, generator=g)
+    gain = torch.tensor([1.3])
+    x0 = x.cpu().clone()
+    want_a = ref.scalar_norm_add(x0, y, gain, 1e-5, dt)
+    got_a = ops.scalar_norm_add(x, y.to(DEV), gain.to(DEV), 1e-5, dt)
+    torch.testing.assert_close(x.cpu(), x0, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(got_a.float().cpu(), want_a.float(), **_tol(dt))
+    fin = ops.scalar_norm_add(x, None, gain.to(DEV), 1e-5, dt)
+    torch.testing.assert_close(fin.float().cpu(), ref.scalar_norm_add(x0, None, gain, 1e-5, dt).float(), **_tol(dt))
+    torch.testing.assert_close(x.cpu(), x0, atol=1e-5, rtol=1e-5)          # untouched without an addend
+    torch.testing.assert_close(ops.relu2(y.to(DEV), dt).float().cpu(), ref.relu2(y, dt).float(), **_tol(dt))
+    rows = torch.tensor([3, 0, 8], dtype=torch.int32)
+    torch.testing.assert_close(ops.gather_rows(x, rows.to(DEV)).cpu(), x0[rows.long()])
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("w", [5, 130])
+def test_mingru_scan(dt, w):
+    g = torch.Generator().manual_seed(w)
+    cu, pos, _ = _seqs([7, 1, 3, 1], [0, 9, 4, 0])
+    slots = torch.tensor([2, 0, -1, 3], dtype=torch.int32)
+    zxg = torch.randn(12, 3 * w, generator=g) * 2
+    st = torch.randn(5, w, generator=g)
+    st_ref = st.clone()
+    want = ref.mingru_scan(zxg, st_ref, cu, pos, slots, dt)
+    st_dev = st.to(DEV)
+    got = ops.mingru_scan(zxg.to(DEV), st_dev, cu.to(DEV), pos.to(DEV), slots.to(DEV), dt)
+    live = torch.tensor([True] * 8 + [False] * 3 + [True])
+    torch.testing.assert_close(got.float().cpu()[live], want.float()[live], **_tol(dt))
+    torch.testing.assert_close(st_dev.cpu(), st_ref, atol=1e-5, rtol=1e-5)     # slot 1 and the skipped sequence untouched
+
+
+@pytest.mark.parametrize("H,D,Dv", [(2, 32, 32), (3, 24, 70), (1, 100, 8)])
+def test_gla_scan_and_headnorm(H, D, Dv):
+    g = torch.Generator().manual_seed(D)
+    cu, pos, _ = _seqs([6, 1, 2], [0, 5, 3])
+    slots = torch.tensor([1, 3, 0], dtype=torch.int32)
+    T = 9
+    proj = torch.randn(T, 2 * H * D + 2 * H * Dv + 5, generator=g)
+    dec = torch.randn(T, H * D, generator=g) * 3
+    st = torch.randn(4, H * D * Dv, generator=g)
+    st_ref = st.clone()
+    want = ref.gla_scan(proj, dec, st_ref, cu, pos, slots, H, D, Dv, 8.0)
+    st_dev = st.to(DEV)
+    pd = proj.to(DEV)
+    got = ops.gla_scan(pd, dec.to(DEV), st_dev, cu.to(DEV), pos.to(DEV), slots.to(DEV), H, D, Dv, 8.0)
+    torch.testing.assert_close(got.cpu(), want, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(st_dev.cpu(), st_ref, atol=1e-4, rtol=1e-4)
+    wn = torch.rand(Dv, generator=g) + 0.5
+    gate = proj[:, 2 * H * D + H * Dv:2 * H * D + 2 * H * Dv]
+    for dt in ACTS:
+        y = ops.headnorm_gate(got, wn.to(DEV), pd[:, 2 * H * D + H * Dv:2 * H * D + 2 * H * Dv], Dv, 1e-5, dt)
+        torch.testing.assert_close(y.float().cpu(), ref.headnorm_gate(want, wn, gate, Dv, 1e-5, dt).float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("H,G,D,Dv,rot,chunk,window", [(4, 2, 32, 20, 8, 7, 0), (3, 3, 48, 72, 48, 0, 5), (2, 1, 16, 16, 0, 0, 0),
+                                                       (6, 2, 96, 40, 24, 100, 0)])
+def test_qkv_prep_and_masked_attention(dt, H, G, D, Dv, rot, chunk, window):
+    g = torch.Generator().manual_seed(H * 100 + D)
+    BS, NB = 16, 24
+    lens, starts = [150, 1, 37], [0, 70, 20]
+    cu, pos, rs = _seqs(lens, starts)
+    T = int(cu[-1])
+    # block tables: distinct shuffled blocks per sequence
+    perm = torch.randperm(NB, generator=g).tolist()
+    need = [(s + n + BS - 1) // BS for n, s in zip(lens, starts)]
+    bt = torch.zeros(3, max(need), dtype=torch.int32)
+    at = 0
+    for b, n in enumerate(need):
+        bt[b, :n] = torch.tensor(perm[at:at + n], dtype=torch.int32)
+        at += n
+    slot = torch.tensor([int(bt[b, p // BS]) * BS + p % BS for b, p in zip(rs.tolist(), pos.tolist())], dtype=torch.int32)
+    kc = torch.randn(NB, G, BS, D, generator=g).to(dt)        # "earlier" keys already in the cache
+    vc = torch.randn(NB, G, BS, Dv, generator=g).to(dt)
+    qkv = torch.randn(T, H * D + G * D + G * Dv + 3, generator=g)
+    qn, kn = torch.rand(H * D, generator=g) + 0.5, torch.rand(G * D, generator=g) + 0.5
+    half = rot // 2
+    inv = torch.tensor([10000.0 ** (-2.0 * j / rot) for j in range(half)] or [0.0])
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    q_ref = ref.qkv_prep(qkv, qn, kn, pos, slot, kc_ref, vc_ref, H, G, D, Dv, rot, 10000.0, 1e-5)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    q = ops.qkv_prep(qkv.to(DEV), qn.to(DEV), kn.to(DEV), inv.to(DEV), pos.to(DEV), slot.to(DEV), kd, vd, H, G, D, Dv,
+                     rot, 10000.0, 1e-5)
+    torch.testing.assert_close(q.cpu(), q_ref, atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(kd.float().cpu(), kc_ref.float(), **_tol(dt))
+    torch.testing.assert_close(vd.float().cpu(), vc_ref.float(), **_tol(dt))
+    # a layer without keys of its own: queries only
+    q2 = ops.qkv_prep(qkv[:, :H * D].contiguous().to(DEV), qn.to(DEV), None, inv.to(DEV), pos.to(DEV), slot.to(DEV),
+                      None, None, H, G, D, Dv, rot, 10000.0, 1e-5)
+    torch.testing.assert_close(q2.cpu(), q_ref, atol=2e-4, rtol=2e-4)
+    want = ref.attn_masked(q_ref, kc_ref, vc_ref, bt, cu, pos, H, G, D, Dv, 0.3, chunk, window, torch.float32)
+    got = ops.attn_masked(q, kd, vd, bt.to(DEV), cu.to(DEV), rs.to(DEV), pos.to(DEV), H, G, D, Dv, 0.3, chunk, window, dt)
+    torch.testing.assert_close(got.float().cpu(), want, **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-4, rtol=2e-4)))
