@@ -127,6 +127,13 @@ def parse_args(argv=None):
                     help="rehearsal on a one-GPU machine: all --gpus ranks use GPU 0, the process group is gloo with "
                          "host-staged tensors (RCCL refuses two ranks on one device), model groups still use the "
                          "peer-to-peer kernels over IPC-mapped memory. Not a measurement: the ranks share the GPU")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the workloads: prefill / decode throughput of the Nidozen hybrid decoder beside a "
+                         "Llama-shaped transformer of equal size (one GPU, random weights)")
+    ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list out of 1k,2k,4k (model width)")
+    ap.add_argument("--hybrid-prompt", type=int, default=2048)
+    ap.add_argument("--hybrid-batch", type=int, default=32)
+    ap.add_argument("--hybrid-new", type=int, default=48)
     ap.add_argument("--in-child", action="store_true", help=argparse.SUPPRESS)
     a = ap.parse_args(argv)
     wl = ALL_WORKLOADS if a.workload.lower() == "all" else "".join(w.strip().upper() for w in a.workload.split(","))
@@ -749,6 +756,10 @@ def run_isolated(ctx: Ctx, a, argv, letter: str, extra_args=(), pick=None):
 def main(argv=None) -> int:
     argv = sys.argv[1:] if argv is None else argv
     a = parse_args(argv)
+    if a.hybrid:
+        from llm_consensus_amd import bench_hybrid
+
+        return bench_hybrid.run(a)
     env_world = os.environ.get("WORLD_SIZE")
     if env_world is None and a.gpus > 1:
         return launch(a, argv)

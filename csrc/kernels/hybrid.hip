@@ -93,16 +93,34 @@ __global__ void relu2_kernel(const float* __restrict__ y, void* __restrict__ out
 // ---------------------------------------------------------------- minGRU
 // zxg [T, 3w]: update-gate logits | candidate pre-activations | output-gate logits.
 // One thread per (sequence, channel); the recurrence runs over the sequence's rows in order.
+// Long portions are cut into segments of seg_len rows that run side by side (blockIdx.z):
+//   mode 1  every segment scans its rows from zero and leaves (product of (1 - z), local result)
+//           in ``carry`` [B, nseg, 2, w];
+//   mode 2  every segment folds the pairs of the segments before it onto the sequence's state
+//           (S <- a S + b is associative), scans its rows again from there and writes the outputs;
+//           the last segment stores the state.
+// mode 0 is the whole sequence in one go (decoded tokens, short portions): nseg = 1, no carry.
 template <bool AF32>
 __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restrict__ state,
                                    const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                   const int32_t* __restrict__ slots, void* __restrict__ out, int w) {
+                                   const int32_t* __restrict__ slots, void* __restrict__ out, int w, int mode,
+                                   int seg_len, float* __restrict__ carry) {
   const int b = blockIdx.y;
+  const int seg = blockIdx.z, nseg = gridDim.z;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int slot = slots[b];
-  const int r0 = cu_q[b], r1 = cu_q[b + 1];
-  if (c >= w || slot < 0 || r1 <= r0) return;
-  float S = positions[r0] == 0 ? 0.f : state[static_cast<size_t>(slot) * w + c];
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (c >= w || slot < 0 || q1 <= q0) return;
+  const int r0 = mode == 0 ? q0 : q0 + seg * seg_len;
+  const int r1 = mode == 0 ? q1 : min(q1, r0 + seg_len);
+  if (r0 >= q1) return;
+  float* cb = carry != nullptr ? carry + static_cast<size_t>(b) * nseg * 2 * w : nullptr;
+  float S = 0.f, A = 1.f;
+  if (mode != 1) {
+    S = positions[q0] == 0 ? 0.f : state[static_cast<size_t>(slot) * w + c];
+    for (int k = 0; k < seg && mode == 2; ++k)
+      S = cb[(static_cast<size_t>(k) * 2) * w + c] * S + cb[(static_cast<size_t>(k) * 2 + 1) * w + c];
+  }
   typename Act<AF32>::type* o = static_cast<typename Act<AF32>::type*>(out);
   for (int t = r0; t < r1; ++t) {
     const float* row = zxg + static_cast<size_t>(t) * 3 * w;
@@ -110,44 +128,72 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
     const float u = row[w + c];
     const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
     S = (1.f - z) * S + z * cand;
-    Act<AF32>::store(o, static_cast<size_t>(t) * w + c, S * siluf_(row[2 * w + c]));
+    if (mode == 1) A *= 1.f - z;
+    else Act<AF32>::store(o, static_cast<size_t>(t) * w + c, S * siluf_(row[2 * w + c]));
   }
-  state[static_cast<size_t>(slot) * w + c] = S;
+  if (mode == 1) {
+    cb[(static_cast<size_t>(seg) * 2) * w + c] = A;
+    cb[(static_cast<size_t>(seg) * 2 + 1) * w + c] = S;
+  } else if (r1 == q1) {
+    state[static_cast<size_t>(slot) * w + c] = S;
+  }
 }
 
 // ---------------------------------------------------------------- gated linear attention
 // proj [T, ld]: q | k | v at columns 0, H*D, 2*H*D; decay [T, H*D] logits. One block per
-// (value-column tile of 64, head, sequence); thread dv keeps column dv of the head's state
-// S [D, Dv] in registers (DMAX >= D). Per token the block stages q, k and the decay in LDS
+// (value-column tile of 64, head, sequence x segment); thread dv keeps column dv of the head's
+// state S [D, Dv] in registers (DMAX >= D). Per token the block stages q, k and the decay in LDS
 // (double buffered: one barrier per token), then S = a * S + k v^T, o = S^T q.
+// Long portions run as segments of seg_len rows side by side, in three passes:
+//   mode 1  each segment scans its rows from zero; its local state goes to ``cs`` [B, nseg, H, D, Dv]
+//           and the product of its decays to ``ca`` [B, nseg, H, D];
+//   (gla_carry_kernel turns the local states into each segment's incoming state, in place)
+//   mode 2  each segment starts from its incoming state, writes its outputs; the last one stores
+//           the sequence's state.
+// mode 0: the whole sequence in one block (decoded tokens, short portions).
 template <int DMAX>
 __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ proj, int ld,
                                                       const float* __restrict__ decay, float* __restrict__ state,
                                                       const int32_t* __restrict__ cu_q,
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
-                                                      int D, int Dv, float inv_tau, float qscale) {
+                                                      int D, int Dv, float inv_tau, float qscale, int mode, int nseg,
+                                                      int seg_len, float* __restrict__ cs, float* __restrict__ ca) {
   __shared__ float sh[2][3][DMAX];
-  const int b = blockIdx.z, h = blockIdx.y;
+  const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
-  const int r0 = cu_q[b], r1 = cu_q[b + 1];
-  if (slot < 0 || r1 <= r0) return;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (slot < 0 || q1 <= q0) return;
+  const int r0 = mode == 0 ? q0 : q0 + seg * seg_len;
+  const int r1 = mode == 0 ? q1 : min(q1, r0 + seg_len);
+  if (r0 >= q1) return;
   const bool live = dv < Dv;
   float S[DMAX];
   float* st = state + (static_cast<size_t>(slot) * H + h) * D * Dv;
-  const bool fresh = positions[r0] == 0;
+  float* seg_s = cs != nullptr ? cs + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D * Dv : nullptr;
+  const float* from = mode == 2 ? seg_s : st;
+  const bool zero = mode == 1 || (mode == 0 && positions[q0] == 0);
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = (!fresh && live && d < D) ? st[static_cast<size_t>(d) * Dv + dv] : 0.f;
+  for (int d = 0; d < DMAX; ++d) S[d] = (!zero && live && d < D) ? from[static_cast<size_t>(d) * Dv + dv] : 0.f;
+  float aprod[(DMAX + 63) / 64];
+#pragma unroll
+  for (int i = 0; i < (DMAX + 63) / 64; ++i) aprod[i] = 1.f;
   auto stage = [&](int t, int buf) {
     const float* row = proj + static_cast<size_t>(t) * ld + h * D;
     const float* drow = decay + static_cast<size_t>(t) * H * D + h * D;
-    for (int d = threadIdx.x; d < D; d += 64) {
-      sh[buf][0][d] = row[d] * qscale;
-      sh[buf][1][d] = row[H * D + d];
-      const float z = drow[d];
-      // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
-      sh[buf][2][d] = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+#pragma unroll
+    for (int i = 0; i < (DMAX + 63) / 64; ++i) {
+      const int d = threadIdx.x + 64 * i;
+      if (d < D) {
+        sh[buf][0][d] = row[d] * qscale;
+        sh[buf][1][d] = row[H * D + d];
+        const float z = drow[d];
+        // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
+        const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+        sh[buf][2][d] = a;
+        aprod[i] *= a;
+      }
     }
   };
   stage(r0, 0);
@@ -164,13 +210,47 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
         o += S[d] * sh[buf][0][d];
       }
     }
-    if (live) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
+    if (live && mode != 1) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
     __syncthreads();
   }
-  if (live) {
+  if (mode == 1) {
+    if (live) {
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < D) seg_s[static_cast<size_t>(d) * Dv + dv] = S[d];
+    }
+    if (blockIdx.x == 0) {
+      float* a = ca + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D;
+#pragma unroll
+      for (int i = 0; i < (DMAX + 63) / 64; ++i)
+        if (threadIdx.x + 64 * i < D) a[threadIdx.x + 64 * i] = aprod[i];
+    }
+  } else if (live && r1 == q1) {
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
       if (d < D) st[static_cast<size_t>(d) * Dv + dv] = S[d];
+  }
+}
+
+// Between the two segment passes: cs[b, s] holds segment s's local state on entry and the state the
+// segment STARTS from on exit (the sequence's own state for s = 0). One thread per state element.
+__global__ void gla_carry_kernel(float* __restrict__ cs, const float* __restrict__ ca, const float* __restrict__ state,
+                                 const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                 const int32_t* __restrict__ slots, int H, int D, int Dv, int nseg, int seg_len) {
+  const int b = blockIdx.y;
+  const size_t n = static_cast<size_t>(H) * D * Dv;
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int slot = slots[b];
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (i >= n || slot < 0 || q1 <= q0) return;
+  const size_t hd = i / Dv;                         // (head, key channel)
+  float carry = positions[q0] == 0 ? 0.f : state[static_cast<size_t>(slot) * n + i];
+  const int used = (q1 - q0 + seg_len - 1) / seg_len;
+  for (int s = 0; s < used; ++s) {
+    float* p = cs + (static_cast<size_t>(b) * nseg + s) * n + i;
+    const float local = *p;
+    *p = carry;
+    carry = ca[(static_cast<size_t>(b) * nseg + s) * H * D + hd] * carry + local;
   }
 }
 
@@ -425,41 +505,77 @@ LC_EXPORT int lc_relu2(const void* y, void* out, int act_f32, long long n, hipSt
   LC_RETURN_LAST_ERROR();
 }
 
+// ``max_len``: the longest portion of the step (host-known). Portions longer than two segments take
+// the segmented passes; ``scratch`` then holds B * nseg * 2 * w floats (see lc_scan_scratch_floats).
+constexpr int kScanSegment = 64;
+
+LC_EXPORT long long lc_scan_scratch_floats(int B, int max_len, long long state_floats, long long decay_floats) {
+  if (max_len <= 2 * kScanSegment) return 0;
+  const long long nseg = (max_len + kScanSegment - 1) / kScanSegment;
+  return static_cast<long long>(B) * nseg * (state_floats + decay_floats);
+}
+
 LC_EXPORT int lc_mingru_scan(const void* zxg, void* state, const void* cu_q, const void* positions, const void* slots,
-                             void* out, int act_f32, int B, int w, hipStream_t st) {
+                             void* out, int act_f32, int B, int w, int max_len, void* scratch, hipStream_t st) {
   if (B <= 0) return 0;
   if (w <= 0) return -1;
-  const dim3 grid((w + 127) / 128, B), block(128);
-  if (act_f32)
-    mingru_scan_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(zxg), static_cast<float*>(state),
-                                                     static_cast<const int32_t*>(cu_q),
-                                                     static_cast<const int32_t*>(positions),
-                                                     static_cast<const int32_t*>(slots), out, w);
-  else
-    mingru_scan_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(zxg), static_cast<float*>(state),
-                                                      static_cast<const int32_t*>(cu_q),
-                                                      static_cast<const int32_t*>(positions),
-                                                      static_cast<const int32_t*>(slots), out, w);
+  const bool segmented = max_len > 2 * kScanSegment;
+  if (segmented && scratch == nullptr) return -1;
+  const int nseg = segmented ? (max_len + kScanSegment - 1) / kScanSegment : 1;
+  const dim3 grid((w + 127) / 128, B, nseg), block(128);
+#define LC_GRU(A32, MODE)                                                                                           \
+  mingru_scan_kernel<A32><<<grid, block, 0, st>>>(static_cast<const float*>(zxg), static_cast<float*>(state),       \
+                                                  static_cast<const int32_t*>(cu_q),                                \
+                                                  static_cast<const int32_t*>(positions),                           \
+                                                  static_cast<const int32_t*>(slots), out, w, MODE, kScanSegment,   \
+                                                  static_cast<float*>(scratch))
+  if (segmented) {
+    LC_GRU(true, 1);
+    if (act_f32) LC_GRU(true, 2);
+    else LC_GRU(false, 2);
+  } else if (act_f32) {
+    LC_GRU(true, 0);
+  } else {
+    LC_GRU(false, 0);
+  }
+#undef LC_GRU
   LC_RETURN_LAST_ERROR();
 }
 
 LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* state, const void* cu_q,
                           const void* positions, const void* slots, void* out, int B, int H, int D, int Dv, float tau,
-                          hipStream_t st) {
+                          int max_len, void* scratch, hipStream_t st) {
   if (B <= 0) return 0;
   if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + H * Dv || !(tau > 0.f)) return -1;
-  const dim3 grid((Dv + 63) / 64, H, B), block(64);
+  const bool segmented = max_len > 2 * kScanSegment;
+  if (segmented && scratch == nullptr) return -1;
+  const int nseg = segmented ? (max_len + kScanSegment - 1) / kScanSegment : 1;
+  const dim3 grid((Dv + 63) / 64, H, B * nseg), block(64);
   const float qscale = 1.f / sqrtf(static_cast<float>(D));
-#define LC_GLA(DMAX)                                                                                                \
+  float* cs = static_cast<float*>(scratch);
+  float* ca = segmented ? cs + static_cast<size_t>(B) * nseg * H * D * Dv : nullptr;
+#define LC_GLA(DMAX, MODE)                                                                                             \
   gla_scan_kernel<DMAX><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, static_cast<const float*>(decay), \
                                                 static_cast<float*>(state), static_cast<const int32_t*>(cu_q),      \
                                                 static_cast<const int32_t*>(positions),                             \
                                                 static_cast<const int32_t*>(slots), static_cast<float*>(out), H, D, \
-                                                Dv, 1.f / tau, qscale)
-  if (D <= 32) LC_GLA(32);
-  else if (D <= 64) LC_GLA(64);
-  else if (D <= 128) LC_GLA(128);
-  else LC_GLA(256);
+                                                Dv, 1.f / tau, qscale, MODE, nseg, kScanSegment, cs, ca)
+#define LC_GLA_D(MODE)          \
+  if (D <= 32) LC_GLA(32, MODE);  \
+  else if (D <= 64) LC_GLA(64, MODE); \
+  else if (D <= 128) LC_GLA(128, MODE); \
+  else LC_GLA(256, MODE)
+  if (segmented) {
+    LC_GLA_D(1);
+    const size_t n = static_cast<size_t>(H) * D * Dv;
+    gla_carry_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256), B), dim3(256), 0, st>>>(
+        cs, ca, static_cast<const float*>(state), static_cast<const int32_t*>(cu_q),
+        static_cast<const int32_t*>(positions), static_cast<const int32_t*>(slots), H, D, Dv, nseg, kScanSegment);
+    LC_GLA_D(2);
+  } else {
+    LC_GLA_D(0);
+  }
+#undef LC_GLA_D
 #undef LC_GLA
   LC_RETURN_LAST_ERROR();
 }

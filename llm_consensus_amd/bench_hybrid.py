@@ -1,0 +1,128 @@
+"""Prefill and decode throughput of the Nidozen hybrid decoder beside a Llama-shaped transformer of
+equal width, depth and head sizes (``bench.py --hybrid``). Random weights, synthetic tokens.
+
+Per size: one prompt of ``prompt`` tokens goes through each engine as a single step (prefill
+tokens/s), then ``batch`` requests decode ``new`` tokens each from recorded steps (decode tokens/s).
+The hybrid stack repeats (attention, minGRU, attention on the first layer's keys, minGRU, gated
+linear attention); the transformer has full causal attention and a SwiGLU feed-forward. Prints one
+JSON line. Per-kernel times come from running this under ``rocprofv3 --kernel-trace --stats``.
+"""
+from __future__ import annotations
+
+import json
+import time
+from typing import Dict
+
+import numpy as np
+import torch
+
+SIZES = {
+    # width, layers, heads, kv heads, head dim, ff, chunk
+    "1k": dict(width=1024, layers=5, heads=8, kv=2, dim=128, ff=4096, chunk=512, vocab=32000),
+    "2k": dict(width=2048, layers=10, heads=16, kv=4, dim=128, ff=8192, chunk=1024, vocab=32000),
+    "4k": dict(width=4096, layers=10, heads=32, kv=8, dim=128, ff=14336, chunk=1024, vocab=32000),
+}
+
+
+def hybrid_config(s: dict):
+    from .models.hybrid import config_from_dict
+
+    def attn(kv_from=None):
+        m = {"heads": s["heads"], "kv_heads": s["kv"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+             "mask": {"size": s["chunk"]}, "rot": {"dims": s["dim"] // 2, "base": 10000.0}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": s["ff"]}}
+    layers = []
+    for i in range(s["layers"]):
+        k = i % 5
+        if k == 0:
+            first = len(layers)
+            layers.append(attn())
+        elif k == 2:
+            layers.append(attn(first))
+        elif k in (1, 3):
+            layers.append({"type": "mingru", "mixer": {"width": s["width"]}, "mlp": {"kind": "dense", "ff": s["ff"]}})
+        else:
+            layers.append({"type": "gla", "mixer": {"heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "tau": 16.0,
+                                                     "rank": 64}, "mlp": {"kind": "dense", "ff": s["ff"]}})
+    return config_from_dict({"architecture": "Nidozen", "vocab": s["vocab"], "width": s["width"],
+                             "norm": {"eps": 1e-5}, "layers": layers}, name="nidozen-bench")
+
+
+def transformer_config(s: dict):
+    from .models.config import ModelConfig
+
+    return ModelConfig("llama-bench", s["vocab"], s["width"], s["layers"], s["heads"], s["kv"], s["dim"], s["ff"],
+                       max_position=8192)
+
+
+def _measure(model, prompt: int, batch: int, new: int, steps: int, warmup: int) -> Dict[str, float]:
+    from ._native import core
+    from .engine.engine import Engine
+
+    blocks = (prompt // 64 + 2) + batch * ((64 + new) // 64 + 2) + 8
+    eng = Engine(model, num_kv_blocks=blocks, block_size=64, max_batch_seqs=max(batch, 4), max_model_len=8192,
+                 enable_prefix_cache=False, name="bench")
+    vocab = model.cfg.vocab_size
+    rng = np.random.default_rng(0)
+    times = []
+    for i in range(warmup + steps):
+        toks = rng.integers(0, vocab, prompt).tolist()
+        rid = eng.replay_open()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.replay_step([(rid, toks, [prompt - 1])])
+        torch.cuda.synchronize()
+        if i >= warmup:
+            times.append(time.perf_counter() - t0)
+        eng.replay_close(rid)
+    out = {"prefill_tokens_per_s": prompt / float(np.median(times)), "prefill_ms": 1e3 * float(np.median(times))}
+    p = core.SamplingParams()
+    p.temperature, p.max_new_tokens, p.ignore_eos = 0.8, new, True
+    dec = []
+    for i in range(2):          # the first pass records the decode graphs
+        for b in range(batch):
+            p.seed = 100 * i + b
+            eng.submit(rng.integers(0, vocab, 64).tolist(), params=p)
+        while eng.sched.num_running < batch and eng.step():
+            pass
+        torch.cuda.synchronize()
+        t0, n0 = time.perf_counter(), eng.metrics.snapshot().get("decode.tokens", 0)
+        eng.run_until_done()
+        torch.cuda.synchronize()
+        dec.append((eng.metrics.snapshot().get("decode.tokens", 0) - n0) / (time.perf_counter() - t0))
+    out["decode_tokens_per_s"] = dec[-1]
+    out["decode_ms_per_step"] = 1e3 * batch / dec[-1]
+    return out
+
+
+def run(a) -> int:
+    from .models.hybrid import HybridModel
+    from .models.transformer import TransformerModel
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    res = {"metric": "prefill / decode tokens per second, Nidozen hybrid beside a Llama-shaped transformer of equal size",
+           "dtype": "bf16", "data": "synthetic tokens, random-init weights", "n_gpus": 1,
+           "prompt": a.hybrid_prompt, "batch": a.hybrid_batch, "new_tokens": a.hybrid_new, "sizes": {}}
+    for name in [n for n in a.hybrid_sizes.split(",") if n]:
+        s = SIZES[name]
+        row = {}
+        for kind in ("nidozen", "llama"):
+            if kind == "nidozen":
+                model = HybridModel.random_init(hybrid_config(s), dev, seed=1)
+            else:
+                model = TransformerModel.random_init(transformer_config(s), dev, seed=1)
+            row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup)
+            row[kind]["weight_gb"] = model.weight_bytes() / 1e9
+            del model
+            torch.cuda.empty_cache()
+        row["prefill_ratio"] = row["nidozen"]["prefill_tokens_per_s"] / row["llama"]["prefill_tokens_per_s"]
+        row["decode_ratio"] = row["nidozen"]["decode_tokens_per_s"] / row["llama"]["decode_tokens_per_s"]
+        res["sizes"][name] = row
+    print(json.dumps(res))
+    if a.out:
+        with open(a.out, "w") as f:
+            f.write(json.dumps(res) + "\n")
+    return 0

@@ -1334,12 +1334,26 @@ class Engine:
                 if plan.ahead:
                     raise RuntimeError("a decode step launched ahead must not record its graph")
                 t_cap = time.perf_counter()
+                # Recording runs the step once for real before it records it, and the replay below
+                # runs it again. Keys and values land in the same places twice; a recurrent state
+                # would advance twice. So the real run sees no state slots (rows without a slot
+                # are skipped by the recurrences), and the slots go up again for the replay.
+                stateful = self.kvm.num_state_slots > 0
+                if stateful:
+                    keep = h["state_slots"].copy()
+                    g.begin_fill()
+                    h["state_slots"][:] = -1
+                    g.upload()
                 if self.use_graphs:
                     g.capture(self, with_dec)
                 elif self.piecewise == "graphs":
                     g.capture_piecewise(self, with_dec)
                 else:
                     g.capture_launch_lists(self, with_dec)
+                if stateful:
+                    g.begin_fill()
+                    h["state_slots"][:] = keep
+                    g.upload()
                 self.metrics.inc("decode.graph_captures")
                 self.metrics.inc("decode.graph_capture_seconds", time.perf_counter() - t_cap)
             g.replay(with_dec)

@@ -362,6 +362,7 @@ class HybridModel:
         self.lm_head: Optional[ops.LinearWeight] = None
         self.layers: List[HybridLayer] = []
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self._max_len = 1
 
     # ------------------------------------------------------------------ construction
     def set_weights(self, get) -> None:
@@ -477,6 +478,8 @@ class HybridModel:
         lay: StepLayout = getattr(meta, "layout", None) or self._decode_layout(meta, token_ids.numel())
         if c.has_state and lay.state_slots is None:
             raise ValueError(f"{c.name}: the step names no state slots (the engine's KV manager must be made with slots)")
+        # the longest portion of the step: long ones are scanned in parallel segments
+        self._max_len = max(1, int(meta.max_q_len)) if meta.is_prefill else 1
         x, xa = ops.embed_rows(token_ids, self.embed, dt, meta.token_feed)
         for i, L in enumerate(self.layers):
             l = L.spec
@@ -484,7 +487,7 @@ class HybridModel:
                 y = self._attention(i, L, xa, positions, slot_mapping, lay, cache)
             elif l.type == "mingru":
                 zxg = ops.linear(xa, L.proj, out_f32=True)
-                y = ops.mingru_scan(zxg, cache.state(i), lay.cu_q, positions, lay.state_slots, dt)
+                y = ops.mingru_scan(zxg, cache.state(i), lay.cu_q, positions, lay.state_slots, dt, self._max_len)
                 y = ops.linear(y, L.out, out_f32=True)
             else:
                 y = self._gla(i, L, xa, positions, lay, cache)
@@ -518,7 +521,7 @@ class HybridModel:
         logits = ops.linear_any(proj[:, 2 * hd + 2 * hv:].contiguous(), L.decay_up) if not L.decay_up.is_packed \
             else ops.linear(proj[:, 2 * hd + 2 * hv:].to(torch.bfloat16).contiguous(), L.decay_up, out_f32=True)
         o = ops.gla_scan(proj, logits, cache.state(i), lay.cu_q, positions, lay.state_slots, l.heads, l.dim, l.vdim,
-                         l.tau)
+                         l.tau, self._max_len)
         y = ops.headnorm_gate(o, L.head_norm, proj[:, 2 * hd + hv:2 * hd + 2 * hv], l.vdim, self.cfg.rms_eps, self.dtype)
         return ops.linear(y, L.out, out_f32=True)
 

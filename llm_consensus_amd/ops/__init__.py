@@ -946,11 +946,19 @@ def relu2(y: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def _scan_scratch(B: int, max_len: int, state_floats: int, decay_floats: int, device) -> Optional[torch.Tensor]:
+    """Carry buffer of the segmented scans (portions longer than two segments of 64 rows run as
+    segments side by side: hybrid.hip), None when the step's portions are short."""
+    n = int(_hip().lib().lc_scan_scratch_floats(B, int(max_len), state_floats, decay_floats))
+    return torch.empty(n, dtype=torch.float32, device=device) if n else None
+
+
 def mingru_scan(zxg: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
-                slots: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+                slots: torch.Tensor, act_dtype: torch.dtype, max_len: int = 1) -> torch.Tensor:
     """minGRU over the step's sequences: zxg fp32 [T, 3w] (update-gate logits | candidate
     pre-activations | output-gate logits), state fp32 [slots, w] (updated in place). Returns
-    S * silu(g) [T, w] in ``act_dtype``."""
+    S * silu(g) [T, w] in ``act_dtype``. ``max_len``: the longest portion of the step (host-known;
+    long portions are scanned in parallel segments)."""
     if not zxg.is_cuda:
         return ref.mingru_scan(zxg, state, cu_q, positions, slots, act_dtype)
     T, w = zxg.shape[0], zxg.shape[1] // 3
@@ -958,16 +966,20 @@ def mingru_scan(zxg: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, posi
         raise ValueError("mingru_scan: fp32 projections [T, 3w] and fp32 state [slots, w]")
     zxg = zxg.contiguous()
     out = torch.empty(T, w, dtype=act_dtype, device=zxg.device)
+    B = slots.numel()
+    scratch = _scan_scratch(B, max_len, w, w, zxg.device)
     _hip().call("lc_mingru_scan", zxg.data_ptr(), state.data_ptr(), cu_q.data_ptr(), positions.data_ptr(),
-                slots.data_ptr(), out.data_ptr(), _f32flag(act_dtype), slots.numel(), w)
+                slots.data_ptr(), out.data_ptr(), _f32flag(act_dtype), B, w, int(max_len), _hip().ptr(scratch))
     return out
 
 
 def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
-             positions: torch.Tensor, slots: torch.Tensor, H: int, D: int, Dv: int, tau: float) -> torch.Tensor:
+             positions: torch.Tensor, slots: torch.Tensor, H: int, D: int, Dv: int, tau: float,
+             max_len: int = 1) -> torch.Tensor:
     """Gated linear attention over the step's sequences. proj fp32 [T, >= 2HD + HDv] holds
     q | k | v in its first columns, decay_logits fp32 [T, HD]; state fp32 [slots, H*D*Dv]
-    (updated in place). Returns the un-normed read-out fp32 [T, H*Dv]."""
+    (updated in place). Returns the un-normed read-out fp32 [T, H*Dv]. ``max_len`` as in
+    ``mingru_scan``."""
     if not proj.is_cuda:
         return ref.gla_scan(proj, decay_logits, state, cu_q, positions, slots, H, D, Dv, tau)
     T = proj.shape[0]
@@ -977,9 +989,11 @@ def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor
         raise ValueError("gla_scan: shapes do not fit the head sizes")
     decay_logits = decay_logits.contiguous()
     out = torch.empty(T, H * Dv, dtype=torch.float32, device=proj.device)
+    B = slots.numel()
+    scratch = _scan_scratch(B, max_len, H * D * Dv, H * D, proj.device)
     _hip().call("lc_gla_scan", proj.data_ptr(), proj.stride(0), decay_logits.data_ptr(), state.data_ptr(),
-                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), slots.numel(), H, D, Dv,
-                float(tau))
+                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), B, H, D, Dv,
+                float(tau), int(max_len), _hip().ptr(scratch))
     return out
 
 

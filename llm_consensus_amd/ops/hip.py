@@ -61,13 +61,14 @@ _SIGNATURES = {
     "lc_embed_rows": [_P, _P, _I, _P, _P, _I, _I, _I, _I, _P, _P, _P],
     "lc_scalar_norm_add": [_P, _P, _P, _F, _P, _I, _I, _I, _P],
     "lc_relu2": [_P, _P, _I, _L, _P],
-    "lc_mingru_scan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "lc_gla_scan": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P],
+    "lc_mingru_scan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
+    "lc_gla_scan": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _P],
     "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
     "lc_qkv_prep": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "lc_gemm_any": [_P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
 }
+_RESTYPES = {"lc_scan_scratch_floats": ([_I, _I, _L, _L], c_longlong)}      # helpers that return no status
 
 _lib = None
 
@@ -88,6 +89,10 @@ def lib() -> ctypes.CDLL:
                 continue
             fn.argtypes = argtypes
             fn.restype = c_int
+        for name, (argtypes, restype) in _RESTYPES.items():
+            fn = getattr(l, name, None)
+            if fn is not None:
+                fn.argtypes, fn.restype = argtypes, restype
         _lib = l
     return _lib
 

@@ -194,7 +194,7 @@ def test_chunk_edges_show_in_the_logits(device, decode_from):
         moved = np.abs(_edge_logits(eng, alt, decode_from) - base).max(-1)
         end = (j // C + 1) * C
         assert (moved[:j] < 1e-5).all() and (moved[min(end, len(toks)):] < 1e-5).all(), j
-        assert (moved[j:min(end, len(toks))] > 1e-3).all(), j
+        assert (moved[j:min(end, len(toks))] > 5e-5).all(), j
 
 
 @pytest.mark.parametrize("device", DEVICES)

@@ -86,6 +86,35 @@ def test_mingru_scan(dt, w):
     torch.testing.assert_close(st_dev.cpu(), st_ref, atol=1e-5, rtol=1e-5)     # slot 1 and the skipped sequence untouched
 
 
+@pytest.mark.parametrize("dt", ACTS)
+def test_scans_of_long_portions_run_in_segments(dt):
+    """Portions longer than two segments of 64 rows take the three-pass form: same results, with a
+    portion that starts from a kept state, one that starts at position 0, a short one and a skipped one."""
+    g = torch.Generator().manual_seed(9)
+    lens, starts = [300, 129, 5, 200], [40, 0, 7, 3]
+    cu, pos, _ = _seqs(lens, starts)
+    slots = torch.tensor([1, 0, 3, -1], dtype=torch.int32)
+    T, w = int(cu[-1]), 70
+    zxg = torch.randn(T, 3 * w, generator=g) * 2
+    st = torch.randn(4, w, generator=g)
+    st_ref = st.clone()
+    want = ref.mingru_scan(zxg, st_ref, cu, pos, slots, dt)
+    sd = st.to(DEV)
+    got = ops.mingru_scan(zxg.to(DEV), sd, cu.to(DEV), pos.to(DEV), slots.to(DEV), dt, max_len=300)
+    torch.testing.assert_close(got.float().cpu()[:434], want.float()[:434], **_tol(dt))
+    torch.testing.assert_close(sd.cpu(), st_ref, atol=1e-5, rtol=1e-5)
+    H, D, Dv = 2, 24, 70
+    proj = torch.randn(T, 2 * H * D + 2 * H * Dv, generator=g)
+    dec = torch.randn(T, H * D, generator=g) * 2 + 3
+    st = torch.randn(4, H * D * Dv, generator=g)
+    st_ref = st.clone()
+    want = ref.gla_scan(proj, dec, st_ref, cu, pos, slots, H, D, Dv, 4.0)
+    sd = st.to(DEV)
+    got = ops.gla_scan(proj.to(DEV), dec.to(DEV), sd, cu.to(DEV), pos.to(DEV), slots.to(DEV), H, D, Dv, 4.0, max_len=300)
+    torch.testing.assert_close(got.cpu()[:434], want[:434], atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(sd.cpu(), st_ref, atol=2e-4, rtol=2e-4)
+
+
 @pytest.mark.parametrize("H,D,Dv", [(2, 32, 32), (3, 24, 70), (1, 100, 8)])
 def test_gla_scan_and_headnorm(H, D, Dv):
     g = torch.Generator().manual_seed(D)
