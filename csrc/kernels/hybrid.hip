@@ -56,23 +56,29 @@ __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* _
 
 // ---------------------------------------------------------------- scalar-gain RMS norm of a sublayer output
 // With y: x += y * rsqrt(mean(y^2) + eps) * gain, xa = x. Without: xa = x * rsqrt(mean(x^2) + eps) * gain.
-template <bool AF32>
-__global__ void scalar_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gain,
-                                       float eps, void* __restrict__ xa, int T, int d) {
-  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (row >= T) return;
+// WAVES = 1: one wave per row, four rows per block (many rows: bandwidth-bound). WAVES = 4: one
+// block per row (decode steps: few rows, latency-bound, so a row is spread over 256 lanes).
+template <bool AF32, int WAVES>
+__global__ __launch_bounds__(256) void scalar_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                              const float* __restrict__ gain, float eps,
+                                                              void* __restrict__ xa, int T, int d) {
+  __shared__ float red[16];
+  constexpr int LANES = 64 * WAVES;
+  const int row = WAVES == 1 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  const int lane = WAVES == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  if (WAVES == 1 && row >= T) return;
   float* xr = x + static_cast<size_t>(row) * d;
   const float* src = y != nullptr ? y + static_cast<size_t>(row) * d : xr;
+  const float g = gain[0];
   float ss = 0.f;
-  for (int c = lane; c < d; c += 64) {
+  for (int c = lane; c < d; c += LANES) {
     const float v = src[c];
     ss += v * v;
   }
-  ss = wave_sum(ss);
-  const float r = gain[0] / sqrtf(ss / static_cast<float>(d) + eps);
+  ss = WAVES == 1 ? wave_sum(ss) : block_sum(ss, red);
+  const float r = g / sqrtf(ss / static_cast<float>(d) + eps);
   typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
-  for (int c = lane; c < d; c += 64) {
+  for (int c = lane; c < d; c += LANES) {
     float v = src[c] * r;
     if (y != nullptr) {
       v += xr[c];
@@ -406,6 +412,146 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
   }
 }
 
+// ---------------------------------------------------------------- attention of prompt portions on the matrix cores
+// fp32 products on the matrix cores (v_mfma_f32_16x16x4_f32: both operands fp32, so scores and
+// weights stay 32-bit as in the row kernel above). A block is four waves = four consecutive tiles
+// of 16 query rows of ONE sequence and ONE query head; key / value tiles of 16 positions are staged
+// in LDS as fp32 once per block and serve all 64 rows. Per key tile and wave:
+//   S = Q K^T   D/4 MFMAs (A: q[row l&15][d + (l>>4)], B: k[key l&15][d + (l>>4)]; S[row 4(l>>4)+r][key l&15])
+//   masking per element (rows of a tile may lie in different chunks), online softmax per row
+//   (the 16 lanes of a row's keys reduce by shuffles), P through LDS into the A layout,
+//   O += P V    4 MFMAs per 16 value columns (B: v[key 4j + (l>>4)][col l&15]).
+// Row strides in LDS are padded so that the 16 rows of an operand fall into different banks.
+constexpr int kTileMaxVT = 16;     // value width up to 256
+
+LC_DEVICE int lds_stride(int n, int want) { return n + ((want - n % 32 + 32) % 32); }
+
+template <bool CF32, bool AF32>
+__global__ __launch_bounds__(256) void attn_tile_kernel(
+    const float* __restrict__ q, const void* __restrict__ kc, const void* __restrict__ vc,
+    const int32_t* __restrict__ block_tables, int MB, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ positions, void* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale,
+    int chunk, int window) {
+  extern __shared__ float lds[];
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  const int row0 = q0 + blockIdx.x * 64;
+  if (row0 >= q1) return;                                   // the same for the whole block
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lr = lane & 15, lk = lane >> 4;
+  const int g = h / (H / G);
+  const int DS = lds_stride(D, 4), VS = lds_stride(Dv, 16);
+  float* Qs = lds;                                          // [4][16][DS]
+  float* Ks = Qs + 64 * DS;                                 // [16][DS]
+  float* Vs = Ks + 16 * DS;                                 // [16][VS]
+  float* Ps = Vs + 16 * VS + wave * 16 * 17;                // [4][16][17]
+  const int nt = Dv / 16;
+  const int32_t* table = block_tables + static_cast<size_t>(b) * MB;
+  const typename Act<CF32>::type* kbase = static_cast<const typename Act<CF32>::type*>(kc);
+  const typename Act<CF32>::type* vbase = static_cast<const typename Act<CF32>::type*>(vc);
+  // queries of the block's rows, scaled (rows past the portion: zero)
+  for (int i = threadIdx.x; i < 64 * D; i += 256) {
+    const int r = i / D, d = i % D;
+    Qs[r * DS + d] = row0 + r < q1 ? q[(static_cast<size_t>(row0 + r) * H + h) * D + d] * scale : 0.f;
+  }
+  const int p0 = positions[row0];                           // rows of a portion are consecutive positions
+  const int nrows = min(64, q1 - row0);
+  auto first_key = [&](int p) {
+    int lo = 0;
+    if (chunk > 0) lo = (p / chunk) * chunk;
+    if (window > 0) lo = max(lo, p - window + 1);
+    return lo;
+  };
+  const int hi = p0 + nrows - 1;
+  const int pw0 = p0 + 16 * wave;                           // position of this wave's first row
+  const int wave_rows = max(0, min(16, nrows - 16 * wave));
+  const int wave_lo = first_key(pw0), wave_hi = pw0 + wave_rows - 1;
+  float m[4], l[4];
+  f32x4 o[kTileMaxVT];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+  }
+#pragma unroll
+  for (int t = 0; t < kTileMaxVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float* Qw = Qs + wave * 16 * DS;
+  for (int j0 = (first_key(p0) / 16) * 16; j0 <= hi; j0 += 16) {
+    __syncthreads();                                        // the previous tile has been consumed (and Qs is written)
+    for (int i = threadIdx.x; i < 16 * D; i += 256) {
+      const int key = i / D, d = i % D, j = j0 + key;
+      float v = 0.f;
+      if (j <= hi) v = Act<CF32>::load(kbase, (static_cast<size_t>(table[j / BS]) * G + g) * BS * D +
+                                                   static_cast<size_t>(j % BS) * D + d);
+      Ks[key * DS + d] = v;
+    }
+    for (int i = threadIdx.x; i < 16 * Dv; i += 256) {
+      const int key = i / Dv, c = i % Dv, j = j0 + key;
+      float v = 0.f;
+      if (j <= hi) v = Act<CF32>::load(vbase, (static_cast<size_t>(table[j / BS]) * G + g) * BS * Dv +
+                                                   static_cast<size_t>(j % BS) * Dv + c);
+      Vs[key * VS + c] = v;
+    }
+    __syncthreads();
+    const bool mine = wave_rows > 0 && j0 <= wave_hi && j0 + 15 >= wave_lo;     // wave-uniform
+    float corr[4] = {1.f, 1.f, 1.f, 1.f};
+    if (mine) {
+      f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+      for (int d = 0; d < D; d += 4)
+        sacc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qw[lr * DS + d + lk], Ks[lr * DS + d + lk], sacc, 0, 0, 0);
+      const int j = j0 + lr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 4 * lk + r;
+        const int prow = pw0 + row;
+        const bool valid = row < wave_rows && j <= prow && j >= first_key(prow);
+        const float sv = valid ? sacc[r] : -INFINITY;
+        float mt = sv;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
+        const float mn = fmaxf(m[r], mt);
+        const float base = mn == -INFINITY ? 0.f : mn;      // nothing visible yet: weights 0, no NaN
+        const float pv = valid ? expf(sv - base) : 0.f;
+        corr[r] = expf(m[r] - base);
+        float ps = pv;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
+        l[r] = l[r] * corr[r] + ps;
+        m[r] = mn;
+        Ps[row * 17 + lr] = pv;
+      }
+    }
+    __syncthreads();                                        // P is in LDS (a wave reads back what all its lanes wrote)
+    if (mine) {
+#pragma unroll
+      for (int t = 0; t < kTileMaxVT; ++t) {
+        if (t < nt) {
+          f32x4 acc = o[t];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] *= corr[r];
+#pragma unroll
+          for (int j4 = 0; j4 < 4; ++j4)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[lr * 17 + 4 * j4 + lk], Vs[(4 * j4 + lk) * VS + t * 16 + lr],
+                                                       acc, 0, 0, 0);
+          o[t] = acc;
+        }
+      }
+    }
+  }
+  typename Act<AF32>::type* dst = static_cast<typename Act<AF32>::type*>(out);
+#pragma unroll
+  for (int t = 0; t < kTileMaxVT; ++t) {
+    if (t < nt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 4 * lk + r;
+        if (row < wave_rows)
+          Act<AF32>::store(dst, (static_cast<size_t>(row0 + 16 * wave + row) * H + h) * Dv + t * 16 + lr, o[t][r] / l[r]);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- shape-agnostic GEMM
 // C[M, N] = A[M, K] W[N, K]^T (+ bias) with fp32 accumulation on the vector ALUs: 64 x 64 tiles,
 // 16-deep slabs in LDS, 4 x 4 outputs per thread. Any M, N, K; A, W and C each fp32 or bf16.
@@ -487,13 +633,16 @@ LC_EXPORT int lc_scalar_norm_add(void* x, const void* y, const void* gain, float
                                  int d, hipStream_t st) {
   if (T <= 0) return 0;
   if (d <= 0) return -1;
-  const dim3 grid((T + 3) / 4), block(256);
-  if (act_f32)
-    scalar_norm_add_kernel<true><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y),
-                                                         static_cast<const float*>(gain), eps, xa, T, d);
-  else
-    scalar_norm_add_kernel<false><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y),
-                                                          static_cast<const float*>(gain), eps, xa, T, d);
+  const bool few = T <= 512;
+  const dim3 grid(few ? T : (T + 3) / 4), block(256);
+#define LC_SN(A32, WAVES)                                                                                       \
+  scalar_norm_add_kernel<A32, WAVES><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y), \
+                                                             static_cast<const float*>(gain), eps, xa, T, d)
+  if (act_f32 && few) LC_SN(true, 4);
+  else if (act_f32) LC_SN(true, 1);
+  else if (few) LC_SN(false, 4);
+  else LC_SN(false, 1);
+#undef LC_SN
   LC_RETURN_LAST_ERROR();
 }
 
@@ -632,6 +781,32 @@ LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int 
   else if (act_f32) LC_ATT(false, true);
   else LC_ATT(false, false);
 #undef LC_ATT
+  LC_RETURN_LAST_ERROR();
+}
+
+// Prompt portions: sequences [0, n_seq) of cu_q, the longest of ``max_len`` rows. Returns -2 when
+// the shape is not one the tile kernel takes (the caller then uses the row kernel for these rows too).
+LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int cache_f32, const void* block_tables,
+                           int MB, const void* cu_q, const void* positions, void* out, int act_f32, int n_seq,
+                           int max_len, int H, int G, int D, int Dv, int BS, float scale, int chunk, int window,
+                           hipStream_t st) {
+  if (n_seq <= 0 || max_len <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0) return -1;
+  if (D % 4 || Dv % 16 || Dv > 16 * kTileMaxVT) return -2;
+  const int DS = D + ((4 - D % 32 + 32) % 32), VS = Dv + ((16 - Dv % 32 + 32) % 32);
+  const size_t lds = (static_cast<size_t>(80) * DS + 16 * VS + 4 * 16 * 17) * sizeof(float);
+  if (lds > 64 * 1024) return -2;
+  const dim3 grid((max_len + 63) / 64, H, n_seq), block(256);
+#define LC_TILE(C32, A32)                                                                                       \
+  attn_tile_kernel<C32, A32><<<grid, block, lds, st>>>(                                                         \
+      static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \
+      static_cast<const int32_t*>(cu_q), static_cast<const int32_t*>(positions), out, H, G, D, Dv, BS, scale,   \
+      chunk, window)
+  if (cache_f32 && act_f32) LC_TILE(true, true);
+  else if (cache_f32) LC_TILE(true, false);
+  else if (act_f32) LC_TILE(false, true);
+  else LC_TILE(false, false);
+#undef LC_TILE
   LC_RETURN_LAST_ERROR();
 }
 

@@ -363,6 +363,7 @@ class HybridModel:
         self.layers: List[HybridLayer] = []
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self._max_len = 1
+        self._portions = (0, 0)
 
     # ------------------------------------------------------------------ construction
     def set_weights(self, get) -> None:
@@ -480,6 +481,10 @@ class HybridModel:
             raise ValueError(f"{c.name}: the step names no state slots (the engine's KV manager must be made with slots)")
         # the longest portion of the step: long ones are scanned in parallel segments
         self._max_len = max(1, int(meta.max_q_len)) if meta.is_prefill else 1
+        # prompt portions come first (sequences and rows), single decoded tokens ride behind them
+        T = token_ids.numel()
+        self._portions = (meta.block_tables.shape[0], meta.prefill_tokens if meta.riders is not None else T) \
+            if meta.is_prefill else (0, 0)
         x, xa = ops.embed_rows(token_ids, self.embed, dt, meta.token_feed)
         for i, L in enumerate(self.layers):
             l = L.spec
@@ -511,7 +516,8 @@ class HybridModel:
                          vc if l.owns_kv else None, l.heads, l.kv_heads, l.dim, l.vdim, l.rot_dims, l.rot_base,
                          self.cfg.rms_eps)
         a = ops.attn_masked(q, kc, vc, lay.block_tables, lay.cu_q, lay.row_seq, positions, l.heads, l.kv_heads, l.dim,
-                            l.vdim, l.scale, l.chunk, l.window, self.dtype)
+                            l.vdim, l.scale, l.chunk, l.window, self.dtype, n_portions=self._portions[0],
+                            portion_rows=self._portions[1], max_len=self._max_len)
         return ops.linear(a, L.out, out_f32=True)
 
     def _gla(self, i: int, L: HybridLayer, xa, positions, lay: StepLayout, cache: HybridCache):

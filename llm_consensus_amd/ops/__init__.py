@@ -1039,14 +1039,31 @@ def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Ten
     return q
 
 
+def attn_tile_ok(D: int, Dv: int) -> bool:
+    """Whether prompt portions of these head widths take the matrix-core kernel (fp32 MFMA tiles:
+    widths in whole MFMA steps, one block's tiles within 64 KB of LDS); otherwise the row kernel."""
+    if D % 4 or Dv % 16 or Dv > 256:
+        return False
+    ds, vs = D + ((4 - D % 32 + 32) % 32), Dv + ((16 - Dv % 32 + 32) % 32)
+    return (80 * ds + 16 * vs + 4 * 16 * 17) * 4 <= 64 * 1024
+
+
+ATTN_TILE_MIN_ROWS = int(os.environ.get("LC_ATTN_TILE_MIN_ROWS", "16"))
+
+
 def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                 cu_q: torch.Tensor, row_seq: torch.Tensor, positions: torch.Tensor, H: int, G: int, D: int, Dv: int,
-                scale: float, chunk: int, window: int, act_dtype: torch.dtype) -> torch.Tensor:
+                scale: float, chunk: int, window: int, act_dtype: torch.dtype, n_portions: int = 0,
+                portion_rows: int = 0, max_len: int = 0) -> torch.Tensor:
     """Attention of fp32 queries [T, H*D] over paged keys / values of widths D / Dv. The row at
     position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
     j > p - window (``window`` > 0), counted from the start of its sequence. ``row_seq`` [T]
-    names each row's sequence (row of ``block_tables``). Serves portions of prompts and single
-    decoded tokens alike; scores, weights and sums are fp32."""
+    names each row's sequence (row of ``block_tables``); scores, weights and sums are fp32.
+
+    Two kernels: the first ``n_portions`` sequences (rows [0, portion_rows), the longest of
+    ``max_len`` rows) are prompt portions and go, 64 rows of a head per block, through fp32 MFMA
+    tiles; the rows behind them (single decoded tokens) and shapes the tiles do not take go
+    through the row kernel, one wave per (row, head)."""
     if not q.is_cuda:
         return ref.attn_masked(q, k_cache, v_cache, block_tables, cu_q, positions, H, G, D, Dv, scale, chunk, window,
                                act_dtype)
@@ -1055,9 +1072,18 @@ def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
         raise ValueError("attn_masked: contiguous fp32 queries, caches of one type")
     if k_cache.shape[1:] != (G, k_cache.shape[2], D) or v_cache.shape[1:] != (G, k_cache.shape[2], Dv):
         raise ValueError("attn_masked: cache planes do not fit the head sizes")
+    if not 0 <= portion_rows <= T or n_portions > block_tables.shape[0]:
+        raise ValueError("attn_masked: the portions exceed the step")
     out = torch.empty(T, H * Dv, dtype=act_dtype, device=q.device)
-    _hip().call("lc_attn_masked", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _f32flag(k_cache.dtype),
-                block_tables.data_ptr(), block_tables.shape[1], row_seq.data_ptr(), positions.data_ptr(),
-                out.data_ptr(), _f32flag(act_dtype), T, H, G, D, Dv, k_cache.shape[2], float(scale), int(chunk),
-                int(window))
+    BS, MB, cf, af = k_cache.shape[2], block_tables.shape[1], _f32flag(k_cache.dtype), _f32flag(act_dtype)
+    first = 0
+    if n_portions > 0 and portion_rows > 0 and max_len >= ATTN_TILE_MIN_ROWS and attn_tile_ok(D, Dv):
+        _hip().call("lc_attn_tile", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf, block_tables.data_ptr(),
+                    MB, cu_q.data_ptr(), positions.data_ptr(), out.data_ptr(), af, int(n_portions), int(max_len), H, G,
+                    D, Dv, BS, float(scale), int(chunk), int(window))
+        first = portion_rows
+    if first < T:
+        _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
+                    block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
+                    out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window))
     return out

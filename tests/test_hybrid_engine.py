@@ -81,6 +81,8 @@ def limit(dtype):
 @pytest.mark.parametrize("name,layers", [
     ("attention", [attn(), attn(heads=3, kv=3, dim=10, vdim=10, rot=10, chunk=7)]),
     ("one kv head, no rotation", [attn(heads=4, kv=1, rot=0, chunk=9)]),
+    ("widths the matrix-core kernel takes", [attn(dim=16, vdim=32, chunk=12), attn(heads=2, kv=1, dim=24, vdim=16, chunk=20,
+                                                                                  ff=0)]),
     ("shared keys", [attn(), attn(kv_from=0, ff=0), gru(), attn(kv_from=0, chunk=4)]),
     ("mingru", [gru(), gru(width=24, ff=36)]),
     ("gla", [gla(), gla(heads=1, dim=20, vdim=5, tau=1.5, rank=3, ff=20)]),
@@ -115,6 +117,16 @@ def test_portions_and_token_by_token_decoding(device, dtype, cuts):
     toks = tokens(70, MIXED["vocab"], 7)
     want = oracle.forward(MIXED, W, toks)
     assert rel_err(replay_alone(eng, toks, cuts), want) < limit(dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_long_portions(device, dtype):
+    """Portions of a few hundred tokens (the recurrences scan them in parallel segments on the GPU),
+    the second one continuing from the state the first one left."""
+    eng, W = build(MIXED, device, dtype)
+    toks = tokens(340, MIXED["vocab"], 13)
+    assert rel_err(replay_alone(eng, toks, [150, 180]), oracle.forward(MIXED, W, toks)) < limit(dtype)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -177,13 +189,28 @@ def _edge_logits(eng, toks, decode_from):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cuts", [[70], [20, 33, 2, 15], [17, 1, 1, 30]])
+def test_portions_on_the_matrix_core_attention(device, dtype, cuts):
+    """Head widths that take the tiled kernel on the GPU: portions that start inside a chunk, cross
+    chunk and page borders, and are shorter than a tile of 16 rows next to longer ones."""
+    cfg = config([attn(dim=16, vdim=16, chunk=12), gru(), attn(kv_from=0, dim=16, vdim=16, chunk=12, ff=0),
+                  attn(heads=2, kv=2, dim=32, vdim=48, chunk=25, rot=32)])
+    eng, W = build(cfg, device, dtype)
+    toks = tokens(70, cfg["vocab"], 17)
+    assert rel_err(replay_alone(eng, toks, cuts), oracle.forward(cfg, W, toks)) < limit(dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("vdim", [24, 16])
 @pytest.mark.parametrize("decode_from", [0, 3])
-def test_chunk_edges_show_in_the_logits(device, decode_from):
+def test_chunk_edges_show_in_the_logits(device, decode_from, vdim):
     """Attention only (nothing else carries a token forward), peaked softmax: a changed token
     moves the logits of the rows of ITS chunk from its position on, and of no other row. Chunk 10
     against pages of 16: the edges fall inside pages and a page border (16, 32) inside chunks."""
     C = 10
-    cfg = config([attn(heads=2, kv=1, chunk=C, scale=3.0, ff=0), attn(kv_from=0, heads=2, kv=1, chunk=C, scale=3.0)])
+    cfg = config([attn(heads=2, kv=1, vdim=vdim, chunk=C, scale=3.0, ff=0),
+                  attn(kv_from=0, heads=2, kv=1, vdim=vdim, chunk=C, scale=3.0)])
     eng, W = build(cfg, device)
     toks = tokens(43, cfg["vocab"], 31)
     base = _edge_logits(eng, toks, decode_from)
