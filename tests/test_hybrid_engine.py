@@ -205,12 +205,12 @@ def test_portions_on_the_matrix_core_attention(device, dtype, cuts):
 @pytest.mark.parametrize("vdim", [24, 16])
 @pytest.mark.parametrize("decode_from", [0, 3])
 def test_chunk_edges_show_in_the_logits(device, decode_from, vdim):
-    """Attention only (nothing else carries a token forward), peaked softmax: a changed token
+    """Attention only (nothing else carries a token forward), a flat softmax: a changed token
     moves the logits of the rows of ITS chunk from its position on, and of no other row. Chunk 10
     against pages of 16: the edges fall inside pages and a page border (16, 32) inside chunks."""
     C = 10
-    cfg = config([attn(heads=2, kv=1, vdim=vdim, chunk=C, scale=3.0, ff=0),
-                  attn(kv_from=0, heads=2, kv=1, vdim=vdim, chunk=C, scale=3.0)])
+    cfg = config([attn(heads=2, kv=1, vdim=vdim, chunk=C, scale=0.8, ff=0),
+                  attn(kv_from=0, heads=2, kv=1, vdim=vdim, chunk=C, scale=0.8)])
     eng, W = build(cfg, device)
     toks = tokens(43, cfg["vocab"], 31)
     base = _edge_logits(eng, toks, decode_from)
