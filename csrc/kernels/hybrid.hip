@@ -148,8 +148,8 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 // ---------------------------------------------------------------- gated linear attention
 // proj [T, ld]: q | k | v at columns 0, H*D, 2*H*D; decay [T, H*D] logits. One block per
 // (value-column tile of 64, head, sequence x segment); thread dv keeps column dv of the head's
-// state S [D, Dv] in registers (DMAX >= D). Per token the block stages q, k and the decay in LDS
-// (double buffered: one barrier per token), then S = a * S + k v^T, o = S^T q.
+// state S [D, Dv] in registers (DMAX >= D). The block stages q, k and the decay of 16 tokens at a
+// time in LDS (one global round trip per 16 tokens), then per token S = a * S + k v^T, o = S^T q.
 // Long portions run as segments of seg_len rows side by side, in three passes:
 //   mode 1  each segment scans its rows from zero; its local state goes to ``cs`` [B, nseg, H, D, Dv]
 //           and the product of its decays to ``ca`` [B, nseg, H, D];
@@ -157,6 +157,8 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 //   mode 2  each segment starts from its incoming state, writes its outputs; the last one stores
 //           the sequence's state.
 // mode 0: the whole sequence in one block (decoded tokens, short portions).
+constexpr int kGlaBatch = 16;     // tokens staged in LDS at a time
+
 template <int DMAX>
 __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ proj, int ld,
                                                       const float* __restrict__ decay, float* __restrict__ state,
@@ -165,7 +167,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
                                                       int D, int Dv, float inv_tau, float qscale, int mode, int nseg,
                                                       int seg_len, float* __restrict__ cs, float* __restrict__ ca) {
-  __shared__ float sh[2][3][DMAX];
+  __shared__ float4 sh[kGlaBatch][DMAX];          // per token and key channel: (q / sqrt(D), k, decay, -)
   const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
@@ -185,39 +187,46 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   float aprod[(DMAX + 63) / 64];
 #pragma unroll
   for (int i = 0; i < (DMAX + 63) / 64; ++i) aprod[i] = 1.f;
-  auto stage = [&](int t, int buf) {
-    const float* row = proj + static_cast<size_t>(t) * ld + h * D;
-    const float* drow = decay + static_cast<size_t>(t) * H * D + h * D;
+  for (int t0 = r0; t0 < r1; t0 += kGlaBatch) {
+    const int nb = min(kGlaBatch, r1 - t0);
+    // this thread's value column for the batch: the loads are in flight while the batch is staged
+    float v[kGlaBatch];
 #pragma unroll
-    for (int i = 0; i < (DMAX + 63) / 64; ++i) {
-      const int d = threadIdx.x + 64 * i;
-      if (d < D) {
-        sh[buf][0][d] = row[d] * qscale;
-        sh[buf][1][d] = row[H * D + d];
-        const float z = drow[d];
-        // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
-        const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
-        sh[buf][2][d] = a;
-        aprod[i] *= a;
-      }
+    for (int i = 0; i < kGlaBatch; ++i)
+      v[i] = (live && i < nb) ? proj[static_cast<size_t>(t0 + i) * ld + 2 * H * D + h * Dv + dv] : 0.f;
+    __syncthreads();                              // the previous batch has been consumed
+    for (int i = threadIdx.x; i < nb * D; i += 64) {
+      const int tok = i / D, d = i - tok * D;
+      const float* row = proj + static_cast<size_t>(t0 + tok) * ld + h * D;
+      const float z = decay[static_cast<size_t>(t0 + tok) * H * D + h * D + d];
+      // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
+      const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+      sh[tok][d] = make_float4(row[d] * qscale, row[H * D + d], a, 0.f);
     }
-  };
-  stage(r0, 0);
-  __syncthreads();
-  for (int t = r0; t < r1; ++t) {
-    const int buf = (t - r0) & 1;
-    if (t + 1 < r1) stage(t + 1, buf ^ 1);
-    const float v = live ? proj[static_cast<size_t>(t) * ld + 2 * H * D + h * Dv + dv] : 0.f;
-    float o = 0.f;
-#pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
-        S[d] = sh[buf][2][d] * S[d] + sh[buf][1][d] * v;
-        o += S[d] * sh[buf][0][d];
-      }
-    }
-    if (live && mode != 1) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
     __syncthreads();
+    if (mode == 1) {
+#pragma unroll
+      for (int i = 0; i < (DMAX + 63) / 64; ++i) {
+        const int d = threadIdx.x + 64 * i;
+        if (d < D)
+          for (int tok = 0; tok < nb; ++tok) aprod[i] *= sh[tok][d].z;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kGlaBatch; ++i) {
+      if (i < nb) {
+        float o = 0.f;
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d) {
+          if (d < D) {
+            const float4 x = sh[i][d];
+            S[d] = x.z * S[d] + x.y * v[i];
+            o += S[d] * x.x;
+          }
+        }
+        if (live && mode != 1) out[static_cast<size_t>(t0 + i) * H * Dv + h * Dv + dv] = o;
+      }
+    }
   }
   if (mode == 1) {
     if (live) {
@@ -416,7 +425,8 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 // fp32 products on the matrix cores (v_mfma_f32_16x16x4_f32: both operands fp32, so scores and
 // weights stay 32-bit as in the row kernel above). A block is four waves = four consecutive tiles
 // of 16 query rows of ONE sequence and ONE query head; key / value tiles of 16 positions are staged
-// in LDS as fp32 once per block and serve all 64 rows. Per key tile and wave:
+// in LDS as fp32 once per block (16-byte loads, the next tile's loads in flight during the current
+// tile's products) and serve all 64 rows. Per key tile and wave:
 //   S = Q K^T   D/4 MFMAs (A: q[row l&15][d + (l>>4)], B: k[key l&15][d + (l>>4)]; S[row 4(l>>4)+r][key l&15])
 //   masking per element (rows of a tile may lie in different chunks), online softmax per row
 //   (the 16 lanes of a row's keys reduce by shuffles), P through LDS into the A layout,
@@ -425,6 +435,43 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 constexpr int kTileMaxVT = 16;     // value width up to 256
 
 LC_DEVICE int lds_stride(int n, int want) { return n + ((want - n % 32 + 32) % 32); }
+
+// Eight consecutive cache elements as they come from memory (converted when they go to LDS, so
+// that the loads of the NEXT tile stay in flight while the current one is computed).
+template <bool CF32>
+struct Raw8 {
+  u32x4 v[CF32 ? 2 : 1];
+};
+
+template <bool CF32>
+LC_DEVICE Raw8<CF32> load_raw8(const void* base, size_t elem, bool on) {
+  Raw8<CF32> r;
+#pragma unroll
+  for (int i = 0; i < (CF32 ? 2 : 1); ++i) r.v[i] = u32x4{0u, 0u, 0u, 0u};
+  if (on) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const char*>(base) + elem * (CF32 ? 4 : 2));
+    r.v[0] = p[0];
+    if (CF32) r.v[CF32 ? 1 : 0] = p[1];
+  }
+  return r;
+}
+
+template <bool CF32>
+LC_DEVICE void store_raw8(const Raw8<CF32>& r, float* dst) {
+  float4* d4 = reinterpret_cast<float4*>(dst);
+  if (CF32) {
+    d4[0] = make_float4(__uint_as_float(r.v[0][0]), __uint_as_float(r.v[0][1]), __uint_as_float(r.v[0][2]),
+                        __uint_as_float(r.v[0][3]));
+    d4[1] = make_float4(__uint_as_float(r.v[CF32 ? 1 : 0][0]), __uint_as_float(r.v[CF32 ? 1 : 0][1]),
+                        __uint_as_float(r.v[CF32 ? 1 : 0][2]), __uint_as_float(r.v[CF32 ? 1 : 0][3]));
+  } else {
+    const u32x4 w = r.v[0];
+    d4[0] = make_float4(__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xffff0000u), __uint_as_float(w[1] << 16),
+                        __uint_as_float(w[1] & 0xffff0000u));
+    d4[1] = make_float4(__uint_as_float(w[2] << 16), __uint_as_float(w[2] & 0xffff0000u), __uint_as_float(w[3] << 16),
+                        __uint_as_float(w[3] & 0xffff0000u));
+  }
+}
 
 template <bool CF32, bool AF32>
 __global__ __launch_bounds__(256) void attn_tile_kernel(
@@ -447,11 +494,9 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   float* Ps = Vs + 16 * VS + wave * 16 * 17;                // [4][16][17]
   const int nt = Dv / 16;
   const int32_t* table = block_tables + static_cast<size_t>(b) * MB;
-  const typename Act<CF32>::type* kbase = static_cast<const typename Act<CF32>::type*>(kc);
-  const typename Act<CF32>::type* vbase = static_cast<const typename Act<CF32>::type*>(vc);
   // queries of the block's rows, scaled (rows past the portion: zero)
   for (int i = threadIdx.x; i < 64 * D; i += 256) {
-    const int r = i / D, d = i % D;
+    const int r = i / D, d = i - r * D;
     Qs[r * DS + d] = row0 + r < q1 ? q[(static_cast<size_t>(row0 + r) * H + h) * D + d] * scale : 0.f;
   }
   const int p0 = positions[row0];                           // rows of a portion are consecutive positions
@@ -466,6 +511,29 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int pw0 = p0 + 16 * wave;                           // position of this wave's first row
   const int wave_rows = max(0, min(16, nrows - 16 * wave));
   const int wave_lo = first_key(pw0), wave_hi = pw0 + wave_rows - 1;
+  // staging: a tile is 16 keys x D (x Dv) elements = 2 D (2 Dv) units of 8; a thread owns up to two of each
+  const int ku = D / 8, vu = Dv / 8;
+  int kkey[2], kcol[2], vkey[2], vcol[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int u = threadIdx.x + 256 * i;
+    kkey[i] = u < 16 * ku ? u / ku : -1;
+    kcol[i] = (u % ku) * 8;
+    vkey[i] = u < 16 * vu ? u / vu : -1;
+    vcol[i] = (u % vu) * 8;
+  }
+  Raw8<CF32> kr[2], vr[2];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int jk = j0 + kkey[i], jv = j0 + vkey[i];
+      const bool kon = kkey[i] >= 0 && jk <= hi, von = vkey[i] >= 0 && jv <= hi;
+      const size_t krow = kon ? (static_cast<size_t>(table[jk / BS]) * G + g) * BS + jk % BS : 0;
+      const size_t vrow = von ? (static_cast<size_t>(table[jv / BS]) * G + g) * BS + jv % BS : 0;
+      kr[i] = load_raw8<CF32>(kc, krow * D + kcol[i], kon);
+      vr[i] = load_raw8<CF32>(vc, vrow * Dv + vcol[i], von);
+    }
+  };
   float m[4], l[4];
   f32x4 o[kTileMaxVT];
 #pragma unroll
@@ -476,67 +544,68 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
 #pragma unroll
   for (int t = 0; t < kTileMaxVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float* Qw = Qs + wave * 16 * DS;
-  for (int j0 = (first_key(p0) / 16) * 16; j0 <= hi; j0 += 16) {
-    __syncthreads();                                        // the previous tile has been consumed (and Qs is written)
-    for (int i = threadIdx.x; i < 16 * D; i += 256) {
-      const int key = i / D, d = i % D, j = j0 + key;
-      float v = 0.f;
-      if (j <= hi) v = Act<CF32>::load(kbase, (static_cast<size_t>(table[j / BS]) * G + g) * BS * D +
-                                                   static_cast<size_t>(j % BS) * D + d);
-      Ks[key * DS + d] = v;
-    }
-    for (int i = threadIdx.x; i < 16 * Dv; i += 256) {
-      const int key = i / Dv, c = i % Dv, j = j0 + key;
-      float v = 0.f;
-      if (j <= hi) v = Act<CF32>::load(vbase, (static_cast<size_t>(table[j / BS]) * G + g) * BS * Dv +
-                                                   static_cast<size_t>(j % BS) * Dv + c);
-      Vs[key * VS + c] = v;
+  int j0 = (first_key(p0) / 16) * 16;
+  fetch(j0);
+  for (; j0 <= hi; j0 += 16) {
+    __syncthreads();                                        // the previous tile has been consumed
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (kkey[i] >= 0) store_raw8<CF32>(kr[i], Ks + kkey[i] * DS + kcol[i]);
+      if (vkey[i] >= 0) store_raw8<CF32>(vr[i], Vs + vkey[i] * VS + vcol[i]);
     }
     __syncthreads();
+    if (j0 + 16 <= hi) fetch(j0 + 16);                      // in flight while this tile is computed
     const bool mine = wave_rows > 0 && j0 <= wave_hi && j0 + 15 >= wave_lo;     // wave-uniform
-    float corr[4] = {1.f, 1.f, 1.f, 1.f};
-    if (mine) {
-      f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
-      for (int d = 0; d < D; d += 4)
-        sacc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qw[lr * DS + d + lk], Ks[lr * DS + d + lk], sacc, 0, 0, 0);
-      const int j = j0 + lr;
+    if (!mine) continue;
+    f32x4 sacc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};      // two chains keep the matrix pipe busy
+    for (int d = 0; d < D; d += 8) {
+      sacc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(Qw[lr * DS + d + lk], Ks[lr * DS + d + lk], sacc[0], 0, 0, 0);
+      sacc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(Qw[lr * DS + d + 4 + lk], Ks[lr * DS + d + 4 + lk], sacc[1], 0, 0, 0);
+    }
+    const int j = j0 + lr;
+    float corr[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = 4 * lk + r;
-        const int prow = pw0 + row;
-        const bool valid = row < wave_rows && j <= prow && j >= first_key(prow);
-        const float sv = valid ? sacc[r] : -INFINITY;
-        float mt = sv;
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * lk + r;
+      const int prow = pw0 + row;
+      const bool valid = row < wave_rows && j <= prow && j >= first_key(prow);
+      const float sv = valid ? sacc[0][r] + sacc[1][r] : -INFINITY;
+      float mt = sv;
 #pragma unroll
-        for (int off = 8; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
-        const float mn = fmaxf(m[r], mt);
-        const float base = mn == -INFINITY ? 0.f : mn;      // nothing visible yet: weights 0, no NaN
-        const float pv = valid ? expf(sv - base) : 0.f;
-        corr[r] = expf(m[r] - base);
-        float ps = pv;
+      for (int off = 8; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
+      const float mn = fmaxf(m[r], mt);
+      const float base = mn == -INFINITY ? 0.f : mn;        // nothing visible yet: weights 0, no NaN
+      const float pv = valid ? expf(sv - base) : 0.f;
+      corr[r] = expf(m[r] - base);
+      float ps = pv;
 #pragma unroll
-        for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
-        l[r] = l[r] * corr[r] + ps;
-        m[r] = mn;
-        Ps[row * 17 + lr] = pv;
+      for (int off = 8; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
+      l[r] = l[r] * corr[r] + ps;
+      m[r] = mn;
+      Ps[row * 17 + lr] = pv;
+    }
+    // P goes from the score layout to the operand layout through this wave's own LDS patch: the
+    // wave's LDS accesses execute in order, the fences keep the compiler from moving them
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float pa[4];
+#pragma unroll
+    for (int j4 = 0; j4 < 4; ++j4) pa[j4] = Ps[lr * 17 + 4 * j4 + lk];
+#pragma unroll
+    for (int t = 0; t < kTileMaxVT; ++t) {
+      if (t < nt) {
+        f32x4 acc = o[t];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] *= corr[r];
+#pragma unroll
+        for (int j4 = 0; j4 < 4; ++j4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[j4], Vs[(4 * j4 + lk) * VS + t * 16 + lr], acc, 0, 0, 0);
+        o[t] = acc;
       }
     }
-    __syncthreads();                                        // P is in LDS (a wave reads back what all its lanes wrote)
-    if (mine) {
-#pragma unroll
-      for (int t = 0; t < kTileMaxVT; ++t) {
-        if (t < nt) {
-          f32x4 acc = o[t];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[r] *= corr[r];
-#pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4)
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[lr * 17 + 4 * j4 + lk], Vs[(4 * j4 + lk) * VS + t * 16 + lr],
-                                                       acc, 0, 0, 0);
-          o[t] = acc;
-        }
-      }
-    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // P is read before the next tile overwrites it
+    __builtin_amdgcn_wave_barrier();
   }
   typename Act<AF32>::type* dst = static_cast<typename Act<AF32>::type*>(out);
 #pragma unroll
@@ -792,7 +861,7 @@ LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int ca
                            hipStream_t st) {
   if (n_seq <= 0 || max_len <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0) return -1;
-  if (D % 4 || Dv % 16 || Dv > 16 * kTileMaxVT) return -2;
+  if (D % 8 || Dv % 16 || Dv > 16 * kTileMaxVT || D > 256) return -2;
   const int DS = D + ((4 - D % 32 + 32) % 32), VS = Dv + ((16 - Dv % 32 + 32) % 32);
   const size_t lds = (static_cast<size_t>(80) * DS + 16 * VS + 4 * 16 * 17) * sizeof(float);
   if (lds > 64 * 1024) return -2;

@@ -1042,7 +1042,7 @@ def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Ten
 def attn_tile_ok(D: int, Dv: int) -> bool:
     """Whether prompt portions of these head widths take the matrix-core kernel (fp32 MFMA tiles:
     widths in whole MFMA steps, one block's tiles within 64 KB of LDS); otherwise the row kernel."""
-    if D % 4 or Dv % 16 or Dv > 256:
+    if D % 8 or Dv % 16 or Dv > 256 or D > 256:
         return False
     ds, vs = D + ((4 - D % 32 + 32) % 32), Dv + ((16 - Dv % 32 + 32) % 32)
     return (80 * ds + 16 * vs + 4 * 16 * 17) * 4 <= 64 * 1024
