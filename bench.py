@@ -131,6 +131,8 @@ def parse_args(argv=None):
                     help="instead of the workloads: prefill / decode throughput of the Nidozen hybrid decoder beside a "
                          "Llama-shaped transformer of equal size (one GPU, random weights)")
     ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list out of 1k,2k,4k (model width)")
+    ap.add_argument("--hybrid-models", default="nidozen,llama", help="which of the two models to run")
+    ap.add_argument("--hybrid-phases", default="prefill,decode", help="which phases to run (for kernel profiles)")
     ap.add_argument("--hybrid-prompt", type=int, default=2048)
     ap.add_argument("--hybrid-batch", type=int, default=32)
     ap.add_argument("--hybrid-new", type=int, default=48)

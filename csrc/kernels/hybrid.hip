@@ -148,8 +148,9 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 // ---------------------------------------------------------------- gated linear attention
 // proj [T, ld]: q | k | v at columns 0, H*D, 2*H*D; decay [T, H*D] logits. One block per
 // (value-column tile of 64, head, sequence x segment); thread dv keeps column dv of the head's
-// state S [D, Dv] in registers (DMAX >= D). The block stages q, k and the decay of 16 tokens at a
-// time in LDS (one global round trip per 16 tokens), then per token S = a * S + k v^T, o = S^T q.
+// state S [D, Dv] in registers (DMAX >= D). q, k and the decay come prepared (gla_prepare_kernel);
+// the block copies 16 tokens of them at a time into LDS (one global round trip per 16 tokens), then
+// per token S = a * S + k v^T, o = S^T q.
 // Long portions run as segments of seg_len rows side by side, in three passes:
 //   mode 1  each segment scans its rows from zero; its local state goes to ``cs`` [B, nseg, H, D, Dv]
 //           and the product of its decays to ``ca`` [B, nseg, H, D];
@@ -159,15 +160,31 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 // mode 0: the whole sequence in one block (decoded tokens, short portions).
 constexpr int kGlaBatch = 16;     // tokens staged in LDS at a time
 
+// Everything the recurrence reads per (token, head, key channel), computed once and in parallel:
+// (q / sqrt(D), k, decay, -) with decay = sigmoid(logit)^(1/tau) = exp(log_sigmoid(logit) / tau).
+__global__ void gla_prepare_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ decay,
+                                   float4* __restrict__ prep, long long n, int HD, float inv_tau, float qscale) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long long t = i / HD;
+  const int c = static_cast<int>(i - t * HD);
+  const float* row = proj + t * ld;
+  const float z = decay[i];
+  // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|))
+  const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+  prep[i] = make_float4(row[c] * qscale, row[HD + c], a, 0.f);
+}
+
 template <int DMAX>
 __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ proj, int ld,
-                                                      const float* __restrict__ decay, float* __restrict__ state,
+                                                      const float4* __restrict__ prep, float* __restrict__ state,
                                                       const int32_t* __restrict__ cu_q,
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
-                                                      int D, int Dv, float inv_tau, float qscale, int mode, int nseg,
-                                                      int seg_len, float* __restrict__ cs, float* __restrict__ ca) {
+                                                      int D, int Dv, int mode, int nseg, int seg_len,
+                                                      float* __restrict__ cs, float* __restrict__ ca) {
   __shared__ float4 sh[kGlaBatch][DMAX];          // per token and key channel: (q / sqrt(D), k, decay, -)
+  __shared__ float vsh[kGlaBatch][64];            // the batch's values, each thread's own column
   const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
@@ -189,19 +206,19 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   for (int i = 0; i < (DMAX + 63) / 64; ++i) aprod[i] = 1.f;
   for (int t0 = r0; t0 < r1; t0 += kGlaBatch) {
     const int nb = min(kGlaBatch, r1 - t0);
-    // this thread's value column for the batch: the loads are in flight while the batch is staged
-    float v[kGlaBatch];
+    __syncthreads();                              // the previous batch has been consumed
+    // this thread's value column for the batch (written and read back by the same thread)
 #pragma unroll
     for (int i = 0; i < kGlaBatch; ++i)
-      v[i] = (live && i < nb) ? proj[static_cast<size_t>(t0 + i) * ld + 2 * H * D + h * Dv + dv] : 0.f;
-    __syncthreads();                              // the previous batch has been consumed
-    for (int i = threadIdx.x; i < nb * D; i += 64) {
-      const int tok = i / D, d = i - tok * D;
-      const float* row = proj + static_cast<size_t>(t0 + tok) * ld + h * D;
-      const float z = decay[static_cast<size_t>(t0 + tok) * H * D + h * D + d];
-      // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|)); the decay is its exponential over tau
-      const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
-      sh[tok][d] = make_float4(row[d] * qscale, row[H * D + d], a, 0.f);
+      vsh[i][threadIdx.x] = (live && i < nb) ? proj[static_cast<size_t>(t0 + i) * ld + 2 * H * D + h * Dv + dv] : 0.f;
+    // plain copies, all independent: the loads of a batch are in flight together
+#pragma unroll
+    for (int tok = 0; tok < kGlaBatch; ++tok) {
+#pragma unroll
+      for (int i = 0; i < (DMAX + 63) / 64; ++i) {
+        const int d = threadIdx.x + 64 * i;
+        if (tok < nb && d < D) sh[tok][d] = prep[(static_cast<size_t>(t0 + tok) * H + h) * D + d];
+      }
     }
     __syncthreads();
     if (mode == 1) {
@@ -212,20 +229,19 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
           for (int tok = 0; tok < nb; ++tok) aprod[i] *= sh[tok][d].z;
       }
     }
+#pragma unroll 1
+    for (int i = 0; i < nb; ++i) {                // rolled: the body (DMAX steps) is what stays in the instruction cache
+      const float v = vsh[i][threadIdx.x];
+      float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < kGlaBatch; ++i) {
-      if (i < nb) {
-        float o = 0.f;
-#pragma unroll
-        for (int d = 0; d < DMAX; ++d) {
-          if (d < D) {
-            const float4 x = sh[i][d];
-            S[d] = x.z * S[d] + x.y * v[i];
-            o += S[d] * x.x;
-          }
+      for (int d = 0; d < DMAX; ++d) {
+        if (d < D) {
+          const float4 x = sh[i][d];
+          S[d] = x.z * S[d] + x.y * v;
+          o += S[d] * x.x;
         }
-        if (live && mode != 1) out[static_cast<size_t>(t0 + i) * H * Dv + h * Dv + dv] = o;
       }
+      if (live && mode != 1) out[static_cast<size_t>(t0 + i) * H * Dv + h * Dv + dv] = o;
     }
   }
   if (mode == 1) {
@@ -760,24 +776,28 @@ LC_EXPORT int lc_mingru_scan(const void* zxg, void* state, const void* cu_q, con
   LC_RETURN_LAST_ERROR();
 }
 
+// ``prep``: T * H * D float4 of scratch for the per-token operands (gla_prepare_kernel).
 LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* state, const void* cu_q,
-                          const void* positions, const void* slots, void* out, int B, int H, int D, int Dv, float tau,
-                          int max_len, void* scratch, hipStream_t st) {
+                          const void* positions, const void* slots, void* out, int T, int B, int H, int D, int Dv,
+                          float tau, int max_len, void* scratch, void* prep, hipStream_t st) {
   if (B <= 0) return 0;
   if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + H * Dv || !(tau > 0.f)) return -1;
   const bool segmented = max_len > 2 * kScanSegment;
-  if (segmented && scratch == nullptr) return -1;
+  if (prep == nullptr || T <= 0 || (segmented && scratch == nullptr)) return -1;
   const int nseg = segmented ? (max_len + kScanSegment - 1) / kScanSegment : 1;
   const dim3 grid((Dv + 63) / 64, H, B * nseg), block(64);
-  const float qscale = 1.f / sqrtf(static_cast<float>(D));
+  const long long n = static_cast<long long>(T) * H * D;
+  gla_prepare_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st>>>(
+      static_cast<const float*>(proj), ld, static_cast<const float*>(decay), static_cast<float4*>(prep), n, H * D,
+      1.f / tau, 1.f / sqrtf(static_cast<float>(D)));
   float* cs = static_cast<float*>(scratch);
   float* ca = segmented ? cs + static_cast<size_t>(B) * nseg * H * D * Dv : nullptr;
 #define LC_GLA(DMAX, MODE)                                                                                             \
-  gla_scan_kernel<DMAX><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, static_cast<const float*>(decay), \
+  gla_scan_kernel<DMAX><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, static_cast<const float4*>(prep), \
                                                 static_cast<float*>(state), static_cast<const int32_t*>(cu_q),      \
                                                 static_cast<const int32_t*>(positions),                             \
                                                 static_cast<const int32_t*>(slots), static_cast<float*>(out), H, D, \
-                                                Dv, 1.f / tau, qscale, MODE, nseg, kScanSegment, cs, ca)
+                                                Dv, MODE, nseg, kScanSegment, cs, ca)
 #define LC_GLA_D(MODE)          \
   if (D <= 32) LC_GLA(32, MODE);  \
   else if (D <= 64) LC_GLA(64, MODE); \

@@ -57,7 +57,7 @@ def transformer_config(s: dict):
                        max_position=8192)
 
 
-def _measure(model, prompt: int, batch: int, new: int, steps: int, warmup: int) -> Dict[str, float]:
+def _measure(model, prompt: int, batch: int, new: int, steps: int, warmup: int, phases=("prefill", "decode")) -> Dict[str, float]:
     from ._native import core
     from .engine.engine import Engine
 
@@ -67,7 +67,8 @@ def _measure(model, prompt: int, batch: int, new: int, steps: int, warmup: int) 
     vocab = model.cfg.vocab_size
     rng = np.random.default_rng(0)
     times = []
-    for i in range(warmup + steps):
+    out: Dict[str, float] = {}
+    for i in range(warmup + steps if "prefill" in phases else 0):
         toks = rng.integers(0, vocab, prompt).tolist()
         rid = eng.replay_open()
         torch.cuda.synchronize()
@@ -77,7 +78,10 @@ def _measure(model, prompt: int, batch: int, new: int, steps: int, warmup: int) 
         if i >= warmup:
             times.append(time.perf_counter() - t0)
         eng.replay_close(rid)
-    out = {"prefill_tokens_per_s": prompt / float(np.median(times)), "prefill_ms": 1e3 * float(np.median(times))}
+    if times:
+        out = {"prefill_tokens_per_s": prompt / float(np.median(times)), "prefill_ms": 1e3 * float(np.median(times))}
+    if "decode" not in phases:
+        return out
     p = core.SamplingParams()
     p.temperature, p.max_new_tokens, p.ignore_eos = 0.8, new, True
     dec = []
@@ -109,17 +113,20 @@ def run(a) -> int:
     for name in [n for n in a.hybrid_sizes.split(",") if n]:
         s = SIZES[name]
         row = {}
-        for kind in ("nidozen", "llama"):
+        phases = tuple(x for x in a.hybrid_phases.split(",") if x)
+        for kind in [k for k in a.hybrid_models.split(",") if k]:
             if kind == "nidozen":
                 model = HybridModel.random_init(hybrid_config(s), dev, seed=1)
             else:
                 model = TransformerModel.random_init(transformer_config(s), dev, seed=1)
-            row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup)
+            row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup, phases)
             row[kind]["weight_gb"] = model.weight_bytes() / 1e9
             del model
             torch.cuda.empty_cache()
-        row["prefill_ratio"] = row["nidozen"]["prefill_tokens_per_s"] / row["llama"]["prefill_tokens_per_s"]
-        row["decode_ratio"] = row["nidozen"]["decode_tokens_per_s"] / row["llama"]["decode_tokens_per_s"]
+        for ph in ("prefill", "decode"):
+            k = ph + "_tokens_per_s"
+            if all(k in row.get(m, {}) for m in ("nidozen", "llama")):
+                row[ph + "_ratio"] = row["nidozen"][k] / row["llama"][k]
         res["sizes"][name] = row
     print(json.dumps(res))
     if a.out:

@@ -991,9 +991,10 @@ def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor
     out = torch.empty(T, H * Dv, dtype=torch.float32, device=proj.device)
     B = slots.numel()
     scratch = _scan_scratch(B, max_len, H * D * Dv, H * D, proj.device)
+    prep = torch.empty(T * H * D * 4, dtype=torch.float32, device=proj.device)     # (q, k, decay, -) per channel
     _hip().call("lc_gla_scan", proj.data_ptr(), proj.stride(0), decay_logits.data_ptr(), state.data_ptr(),
-                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), B, H, D, Dv,
-                float(tau), int(max_len), _hip().ptr(scratch))
+                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), T, B, H, D, Dv,
+                float(tau), int(max_len), _hip().ptr(scratch), prep.data_ptr())
     return out
 
 

@@ -62,7 +62,7 @@ _SIGNATURES = {
     "lc_scalar_norm_add": [_P, _P, _P, _F, _P, _I, _I, _I, _P],
     "lc_relu2": [_P, _P, _I, _L, _P],
     "lc_mingru_scan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
-    "lc_gla_scan": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _P],
+    "lc_gla_scan": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
     "lc_qkv_prep": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
