@@ -741,12 +741,6 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
     out[static_cast<size_t>(row) * DH + lane + 64 * i] = f32_to_bf16(acc[i] * inv);
 }
 
-__global__ void fill_f32_kernel(float* __restrict__ p, float v, size_t n) {
-  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < n;
-       i += static_cast<size_t>(gridDim.x) * blockDim.x)
-    p[i] = v;
-}
-
 int ilog2(int x) {
   int l = 0;
   while ((1 << l) < x) ++l;
@@ -863,12 +857,5 @@ LC_EXPORT int lc_attn_merge(const void* part_o, const void* part_lse, void* out,
     attn_merge_kernel<64><<<grid, block, 0, stream>>>(static_cast<const float*>(part_o),
                                                       static_cast<const float*>(part_lse),
                                                       static_cast<bf16_t*>(out), np_total, n_rows);
-  LC_RETURN_LAST_ERROR();
-}
-
-LC_EXPORT int lc_fill_f32(void* p, float v, long long n, hipStream_t stream) {
-  if (n <= 0) return 0;
-  const int grid = static_cast<int>(std::min<long long>((n + 255) / 256, 2048));
-  fill_f32_kernel<<<dim3(grid), dim3(256), 0, stream>>>(static_cast<float*>(p), v, static_cast<size_t>(n));
   LC_RETURN_LAST_ERROR();
 }

@@ -307,3 +307,20 @@ LC_EXPORT int lc_l2_normalize(const void* x, void* y, int rows, int d, hipStream
   l2_normalize_kernel<<<dim3(rows), dim3(256), 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(y), d);
   LC_RETURN_LAST_ERROR();
 }
+
+// Fill of 32-bit words (cache pools, flags, scratch: also inside recorded steps, where a
+// memset node must not be used). Lives with the row kernels because every model family needs it.
+namespace {
+__global__ void fill_f32_kernel(float* __restrict__ p, float v, size_t n) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x)
+    p[i] = v;
+}
+}  // namespace
+
+LC_EXPORT int lc_fill_f32(void* p, float v, long long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int grid = static_cast<int>(std::min<long long>((n + 255) / 256, 2048));
+  fill_f32_kernel<<<dim3(grid), dim3(256), 0, stream>>>(static_cast<float*>(p), v, static_cast<size_t>(n));
+  LC_RETURN_LAST_ERROR();
+}
