@@ -149,7 +149,6 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 // proj [T, ld]: q | k | v at columns 0, H*D, 2*H*D; decay [T, H*D] logits. One block per
 // (value-column tile of 64, head, sequence x segment); thread dv keeps column dv of the head's
 // state S [D, Dv] in registers (DMAX >= D). q, k and the decay come prepared (gla_prepare_kernel);
-// the block copies 16 tokens of them at a time into LDS (one global round trip per 16 tokens), then
 // per token S = a * S + k v^T, o = S^T q.
 // Long portions run as segments of seg_len rows side by side, in three passes:
 //   mode 1  each segment scans its rows from zero; its local state goes to ``cs`` [B, nseg, H, D, Dv]
@@ -158,8 +157,6 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 //   mode 2  each segment starts from its incoming state, writes its outputs; the last one stores
 //           the sequence's state.
 // mode 0: the whole sequence in one block (decoded tokens, short portions).
-constexpr int kGlaBatch = 16;     // tokens staged in LDS at a time
-
 // Everything the recurrence reads per (token, head, key channel), computed once and in parallel:
 // (q / sqrt(D), k, decay, -) with decay = sigmoid(logit)^(1/tau) = exp(log_sigmoid(logit) / tau).
 __global__ void gla_prepare_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ decay,
@@ -183,8 +180,6 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
                                                       int D, int Dv, int mode, int nseg, int seg_len,
                                                       float* __restrict__ cs, float* __restrict__ ca) {
-  __shared__ float4 sh[kGlaBatch][DMAX];          // per token and key channel: (q / sqrt(D), k, decay, -)
-  __shared__ float vsh[kGlaBatch][64];            // the batch's values, each thread's own column
   const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
@@ -204,45 +199,45 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   float aprod[(DMAX + 63) / 64];
 #pragma unroll
   for (int i = 0; i < (DMAX + 63) / 64; ++i) aprod[i] = 1.f;
-  for (int t0 = r0; t0 < r1; t0 += kGlaBatch) {
-    const int nb = min(kGlaBatch, r1 - t0);
-    __syncthreads();                              // the previous batch has been consumed
-    // this thread's value column for the batch (written and read back by the same thread)
+  // Lane j of the wave loads the prepared operands of key channels j, j + 64, ... of the token (one
+  // coalesced 16-byte load per lane, the next token's in flight during the current one); the
+  // channel loop then broadcasts them lane by lane (v_readlane) to meet every lane's state column.
+  // No LDS, no barrier.
+  constexpr int NCH = (DMAX + 63) / 64;
+  float4 cur[NCH], nxt[NCH];
+  float vcur, vnxt = 0.f;
+  auto fetch = [&](int t, float4* dst, float& vv) {
+    const float4* x = prep + (static_cast<size_t>(t) * H + h) * D;
 #pragma unroll
-    for (int i = 0; i < kGlaBatch; ++i)
-      vsh[i][threadIdx.x] = (live && i < nb) ? proj[static_cast<size_t>(t0 + i) * ld + 2 * H * D + h * Dv + dv] : 0.f;
-    // plain copies, all independent: the loads of a batch are in flight together
-#pragma unroll
-    for (int tok = 0; tok < kGlaBatch; ++tok) {
-#pragma unroll
-      for (int i = 0; i < (DMAX + 63) / 64; ++i) {
-        const int d = threadIdx.x + 64 * i;
-        if (tok < nb && d < D) sh[tok][d] = prep[(static_cast<size_t>(t0 + tok) * H + h) * D + d];
-      }
+    for (int i = 0; i < NCH; ++i) {
+      const int d = threadIdx.x + 64 * i;
+      dst[i] = d < D ? x[d] : make_float4(0.f, 0.f, 1.f, 0.f);
     }
-    __syncthreads();
-    if (mode == 1) {
+    vv = live ? proj[static_cast<size_t>(t) * ld + 2 * H * D + h * Dv + dv] : 0.f;
+  };
+  fetch(r0, nxt, vnxt);
+  for (int t = r0; t < r1; ++t) {
 #pragma unroll
-      for (int i = 0; i < (DMAX + 63) / 64; ++i) {
-        const int d = threadIdx.x + 64 * i;
-        if (d < D)
-          for (int tok = 0; tok < nb; ++tok) aprod[i] *= sh[tok][d].z;
-      }
-    }
-#pragma unroll 1
-    for (int i = 0; i < nb; ++i) {                // rolled: the body (DMAX steps) is what stays in the instruction cache
-      const float v = vsh[i][threadIdx.x];
-      float o = 0.f;
+    for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+    vcur = vnxt;
+    if (t + 1 < r1) fetch(t + 1, nxt, vnxt);
+    float o = 0.f;
 #pragma unroll
-      for (int d = 0; d < DMAX; ++d) {
-        if (d < D) {
-          const float4 x = sh[i][d];
-          S[d] = x.z * S[d] + x.y * v;
-          o += S[d] * x.x;
+    for (int i = 0; i < NCH; ++i) {
+      aprod[i] *= cur[i].z;                       // this lane's channel of the segment's decay product
+#pragma unroll
+      for (int j = 0; j < 64; ++j) {
+        const int d = 64 * i + j;
+        if (d < DMAX && d < D) {
+          const float qd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cur[i].x), j));
+          const float kd = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cur[i].y), j));
+          const float ad = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cur[i].z), j));
+          S[d] = ad * S[d] + kd * vcur;
+          o += S[d] * qd;
         }
       }
-      if (live && mode != 1) out[static_cast<size_t>(t0 + i) * H * Dv + h * Dv + dv] = o;
     }
+    if (live && mode != 1) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
   }
   if (mode == 1) {
     if (live) {
@@ -406,7 +401,19 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
       crow = (table[j / BS] * G + g) * BS + (j % BS);
       const typename Act<CF32>::type* kr = kbase + static_cast<size_t>(crow) * D;
       float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += qs[d] * Act<CF32>::load(kr, d);
+      if (!CF32 && D % 8 == 0) {
+        // a bf16 key row in 16-byte pieces (rows start on 16-byte borders when D is a multiple of 8)
+        const u32x4* kv = reinterpret_cast<const u32x4*>(kr);
+        for (int c = 0; c < D / 8; ++c) {
+          const u32x4 w = kv[c];
+          const float* qc = qs + 8 * c;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            dot += qc[2 * e] * __uint_as_float(w[e] << 16) + qc[2 * e + 1] * __uint_as_float(w[e] & 0xffff0000u);
+        }
+      } else {
+        for (int d = 0; d < D; ++d) dot += qs[d] * Act<CF32>::load(kr, d);
+      }
       s = dot;
     }
     const float mt = fmaxf(m, wave_max(s));
