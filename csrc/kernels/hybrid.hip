@@ -311,11 +311,19 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(
     void* __restrict__ kc, void* __restrict__ vc, float* __restrict__ q_out, int H, int G, int D, int Dv, int BS,
     int rot_dims, float eps, int has_kv) {
   __shared__ float red[16];
+  __shared__ float cs_tab[2][128];                 // cos / sin of the token's angles (rot_dims / 2 <= 128 of them)
   const int t = blockIdx.x;
   const float* row = qkv + static_cast<size_t>(t) * ld;
   const float pos = static_cast<float>(positions[t]);
   const int half = rot_dims >> 1;
   const int nq = H * D, nk = G * D;
+  const bool tab = half <= 128;                    // the same angles serve every head: computed once per token
+  if (tab)
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      const float ang = pos * inv_freq[j];
+      cs_tab[0][j] = cosf(ang);
+      cs_tab[1][j] = sinf(ang);
+    }                                               // (published by the barriers of the reductions below)
   float ssq = 0.f, ssk = 0.f;
   for (int i = threadIdx.x; i < nq; i += blockDim.x) ssq += row[i] * row[i];
   if (has_kv)
@@ -327,8 +335,15 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(
     const float a = src[idx] * r * w[idx];
     if (i >= rot_dims) return a;
     const int j = i < half ? i : i - half;
-    const float ang = pos * inv_freq[j];
-    const float c = cosf(ang), s = sinf(ang);
+    float c, s;
+    if (tab) {
+      c = cs_tab[0][j];
+      s = cs_tab[1][j];
+    } else {
+      const float ang = pos * inv_freq[j];
+      c = cosf(ang);
+      s = sinf(ang);
+    }
     if (i < half) return a * c - src[idx + half] * r * w[idx + half] * s;
     return a * c + src[idx - half] * r * w[idx - half] * s;
   };
@@ -430,6 +445,7 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
       const int c = lane + 64 * i;
       if (c < Dv) {
         float a = acc[i] * corr;
+#pragma unroll 8                                    // eight value loads in flight at a time
         for (int jj = 0; jj < n; ++jj) a += ps[jj] * Act<CF32>::load(vbase, static_cast<size_t>(rows[jj]) * Dv + c);
         acc[i] = a;
       }
