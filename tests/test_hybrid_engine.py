@@ -89,9 +89,23 @@ def limit(dtype):
 ])
 def test_each_mechanism_whole_prompt(device, dtype, name, layers):
     cfg = config(layers)
+    _whole_prompt(cfg, device, dtype, name)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_depths_the_mfma_products_take(device, dtype):
+    """Width 64 and feed-forward 128: in bf16 on the GPU these projections go through the packed
+    MFMA kernels (depth a multiple of 64, fp32 epilogue), the decay bottleneck (depth 6) does not."""
+    cfg = config([attn(dim=16, vdim=16, ff=128), gru(width=64, ff=64), gla(heads=2, dim=32, vdim=32, ff=128),
+                  attn(kv_from=0, dim=16, vdim=16, ff=0)], width=64, vocab=70)
+    _whole_prompt(cfg, device, dtype, "mfma depths", cuts=[40, 2, 17])
+
+
+def _whole_prompt(cfg, device, dtype, name, cuts=None):
     eng, W = build(cfg, device, dtype)
-    toks = tokens(45, cfg["vocab"], 3)
-    got = replay_alone(eng, toks, [len(toks)])
+    toks = tokens(45 if cuts is None else sum(cuts) + 3, cfg["vocab"], 3)
+    got = replay_alone(eng, toks, cuts or [len(toks)])
     assert rel_err(got, oracle.forward(cfg, W, toks)) < limit(dtype), name
 
 
