@@ -662,10 +662,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
 
 // ---------------------------------------------------------------- shape-agnostic GEMM
 // C[M, N] = A[M, K] W[N, K]^T (+ bias) with fp32 accumulation on the vector ALUs: 64 x 64 tiles,
-// 16-deep slabs in LDS, 4 x 4 outputs per thread. Any M, N, K; A, W and C each fp32 or bf16.
+// 16-deep slabs in LDS, 4 x 4 outputs per thread. Any M, N, K; A, W and C each fp32 or bf16; A may be
+// a column slice (row stride lda).
 // epi 1: square of relu.
 template <bool AF32, bool WF32, bool CF32>
-__global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ A, const void* __restrict__ W,
+__global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ A, int lda, const void* __restrict__ W,
                                                        const void* __restrict__ bias, void* __restrict__ C, int M, int N,
                                                        int K, int epi) {
   __shared__ float As[16][64 + 4];
@@ -678,7 +679,7 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ 
   for (int k0 = 0; k0 < K; k0 += 16) {
     for (int i = threadIdx.x; i < 64 * 16; i += 256) {
       const int r = i >> 4, k = i & 15;
-      As[k][r] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * K + k0 + k) : 0.f;
+      As[k][r] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * lda + k0 + k) : 0.f;
       Ws[k][r] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
     }
     __syncthreads();
@@ -922,12 +923,13 @@ LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int ca
   LC_RETURN_LAST_ERROR();
 }
 
-LC_EXPORT int lc_gemm_any(const void* A, int a_f32, const void* W, int w_f32, const void* bias, void* C, int c_f32,
-                          int M, int N, int K, int epi, hipStream_t st) {
+// A may be a column slice of a wider matrix: ``lda`` is its row stride in elements.
+LC_EXPORT int lc_gemm_any(const void* A, int a_f32, int lda, const void* W, int w_f32, const void* bias, void* C,
+                          int c_f32, int M, int N, int K, int epi, hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0) return -1;
+  if (K <= 0 || lda < K) return -1;
   const dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
-#define LC_GA(A32, W32, C32) gemm_any_kernel<A32, W32, C32><<<grid, block, 0, st>>>(A, W, bias, C, M, N, K, epi)
+#define LC_GA(A32, W32, C32) gemm_any_kernel<A32, W32, C32><<<grid, block, 0, st>>>(A, lda, W, bias, C, M, N, K, epi)
   const int sel = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
   switch (sel) {
     case 0: LC_GA(false, false, false); break;

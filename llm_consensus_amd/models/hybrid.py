@@ -410,7 +410,9 @@ class HybridModel:
                 out = lin(load(m + "o"))
             else:
                 proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "a1")], 0))
-                kw["decay_up"] = lin(load(m + "a2"), load(m + "a2.b"))
+                # the bottleneck's output is an fp32 column slice of the fused projection: the small
+                # second product takes it as it is through the shape-agnostic kernel
+                kw["decay_up"] = ops.LinearWeight.from_dense(load(m + "a2"), load(m + "a2.b"), dev, dtype=dt, plain=True)
                 kw["head_norm"] = f32(load(m + "norm"))
                 out = lin(load(m + "o"))
             if l.ff:
@@ -524,8 +526,7 @@ class HybridModel:
         l = L.spec
         hd, hv = l.heads * l.dim, l.heads * l.vdim
         proj = ops.linear(xa, L.proj, out_f32=True)                 # q | k | v | gate | bottleneck
-        logits = ops.linear_any(proj[:, 2 * hd + 2 * hv:].contiguous(), L.decay_up) if not L.decay_up.is_packed \
-            else ops.linear(proj[:, 2 * hd + 2 * hv:].to(torch.bfloat16).contiguous(), L.decay_up, out_f32=True)
+        logits = ops.linear_any(proj[:, 2 * hd + 2 * hv:], L.decay_up)
         o = ops.gla_scan(proj, logits, cache.state(i), lay.cu_q, positions, lay.state_slots, l.heads, l.dim, l.vdim,
                          l.tau, self._max_len)
         y = ops.headnorm_gate(o, L.head_norm, proj[:, 2 * hd + hv:2 * hd + 2 * hv], l.vdim, self.cfg.rms_eps, self.dtype)

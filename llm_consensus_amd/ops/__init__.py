@@ -120,7 +120,7 @@ class LinearWeight:
 
     @classmethod
     def from_dense(cls, W: torch.Tensor, bias: Optional[torch.Tensor] = None, device=None, swiglu: bool = False,
-                   dtype: torch.dtype = torch.bfloat16, any_shape: bool = False):
+                   dtype: torch.dtype = torch.bfloat16, any_shape: bool = False, plain: bool = False):
         """W row-major [N, K] in final row order (already interleaved when swiglu). With
         ``any_shape`` a weight the MFMA kernels do not take (fp32, or a reduction depth that is
         no multiple of 64) stays row-major on the GPU too and goes through the shape-agnostic
@@ -129,7 +129,8 @@ class LinearWeight:
         N, K = W.shape
         W = W.to(device=device, dtype=dtype)
         b = bias.to(device=device, dtype=dtype).contiguous() if bias is not None else None
-        plain = any_shape and (dtype != torch.bfloat16 or K % 64 != 0)
+        # ``plain``: row-major whatever the shape (small products whose input is an fp32 column slice)
+        plain = plain or (any_shape and (dtype != torch.bfloat16 or K % 64 != 0))
         if plain and swiglu:
             raise ValueError("the shape-agnostic product has no SwiGLU epilogue")
         data = pack_weight(W) if (device.type == "cuda" and not plain) else W.contiguous()
@@ -891,9 +892,11 @@ def linear_any(x: torch.Tensor, w: LinearWeight, out_f32: bool = True, epi_relu2
         return (torch.relu(y).pow(2) if epi_relu2 else y).to(odt)
     if w.is_packed:
         raise ValueError("linear_any takes row-major weights")
-    x = x.contiguous()
+    if x.stride(1) != 1:
+        x = x.contiguous()              # (a column slice of a wider matrix is taken as it is)
     y = torch.empty(M, w.n, dtype=odt, device=x.device)
-    _hip().call("lc_gemm_any", x.data_ptr(), _f32flag(x.dtype), w.data.data_ptr(), _f32flag(w.data.dtype),
+    _hip().call("lc_gemm_any", x.data_ptr(), _f32flag(x.dtype), x.stride(0) if M > 1 else max(x.stride(0), w.k),
+                w.data.data_ptr(), _f32flag(w.data.dtype),
                 _hip().ptr(w.bias), y.data_ptr(), 1 if out_f32 else 0, M, w.n, w.k, 1 if epi_relu2 else 0)
     return y
 

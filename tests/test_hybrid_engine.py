@@ -294,3 +294,34 @@ def test_requests_the_family_does_not_serve_are_refused(device):
         eng.submit([1, 2, 3], kind=core.RequestKind.Embed)
     with pytest.raises(ValueError):
         eng.submit([1, 2, 3], n=2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_serving_steps_launch_only_the_kernel_library(dtype):
+    """Prompt portions, mixed steps, decode steps and replayed steps of a hybrid model: PyTorch
+    launches no kernel of its own in any of them (allocations, views and buffer copies aside)."""
+    from llm_consensus_amd.utils.audit import AtenAudit
+
+    cfg = config([attn(dim=16, vdim=16, ff=128), gru(width=64, ff=64), gla(heads=2, dim=32, vdim=32, ff=0),
+                  attn(kv_from=0, dim=16, vdim=16, ff=0), attn(heads=2, kv=1, dim=12, vdim=24)], width=64, vocab=70)
+    eng, _ = build(cfg, "cuda:0", dtype, blocks=40, slots=3, max_batch_seqs=3, max_prefill_tokens=24)
+    p = core.SamplingParams()
+    p.temperature, p.max_new_tokens, p.ignore_eos = 0.7, 5, True
+
+    def work():
+        rids = [eng.submit(tokens(n, cfg["vocab"], n), params=p) for n in (30, 5, 41)]
+        eng.run_until_done()
+        rid = eng.replay_open()
+        eng.replay_step([(rid, tokens(20, cfg["vocab"], 1), [0, 19])])
+        eng.replay_step([(rid, [3], [0])])
+        eng.replay_close(rid)
+        return [eng.pop_result(r) for r in rids]
+
+    work()                                   # first use: lazy initialisation happens here
+    torch.cuda.synchronize()
+    with AtenAudit() as audit:
+        outs = work()
+        torch.cuda.synchronize()
+    assert all(len(o.token_ids[0]) == 5 for o in outs)
+    assert audit.kernels == {}, audit.kernels
