@@ -110,7 +110,12 @@ def default_device() -> torch.device:
 
 
 def model_config_of(spec: ModelSpec):
-    return from_hf_config(spec.path) if spec.path else get_preset(spec.preset or "tiny-llama")
+    """The configuration of a model spec: of its checkpoint's family (models/registry.py) or of a preset."""
+    if spec.path:
+        from .models.registry import resolve
+
+        return resolve(spec.path).read_config(spec.path)
+    return get_preset(spec.preset or "tiny-llama")
 
 
 def build_backend(spec: ModelSpec, device: torch.device, comm=None, tp_rank: int = 0) -> EngineBackend:
@@ -120,7 +125,10 @@ def build_backend(spec: ModelSpec, device: torch.device, comm=None, tp_rank: int
     tp_size = spec.tp if grouped else 1
     model = build_model(spec, device, tp_rank=tp_rank if tp_size > 1 else 0, tp_size=tp_size, comm=comm,
                         ep_size=spec.ep if grouped else 1, ep_mode=spec.ep_mode)
-    max_len = min(model.cfg.max_position, spec.max_model_len) if spec.max_model_len > 0 else model.cfg.max_position
+    # (a design without a position limit reports a very large one: the step buffers are sized by
+    # the longest sequence SERVED, so an unconfigured limit falls back to 8192 tokens there)
+    max_len = min(model.cfg.max_position, spec.max_model_len) if spec.max_model_len > 0 \
+        else min(model.cfg.max_position, 8192 if model.cfg.max_position > (1 << 17) else model.cfg.max_position)
     eng = Engine(model, block_size=spec.kv_block_size if device.type == "cuda" else 16,
                  max_batch_seqs=spec.max_batch_seqs, max_prefill_tokens=spec.max_prefill_tokens,
                  max_model_len=max_len, kv_fraction=spec.kv_fraction,

@@ -103,6 +103,9 @@ class HybridConfig:
     def kv_elems_per_token(self) -> int:
         return sum(l.kv_heads * (l.dim + l.vdim) for l in self.layers if l.owns_kv)
 
+    def kv_bytes_per_token(self, bytes_per_elem: int = 2) -> int:
+        return self.kv_elems_per_token() * bytes_per_elem
+
     def state_floats(self) -> int:
         return sum(l.state_size() for l in self.layers)
 

@@ -157,6 +157,27 @@ def load_hybrid(path: str, device, dtype=torch.bfloat16):
     return model
 
 
+def write_random_hybrid_checkpoint(cfg, path: str, seed: int = 0) -> Path:
+    """Writes a hybrid decoder's checkpoint directory (``config.json`` + ``model.safetensors``,
+    bf16) with random weights of the configured shapes: test helper and offline stand-in."""
+    from safetensors.torch import save_file
+
+    from .hybrid import HybridModel, config_to_dict, param_shapes
+
+    out = Path(path)
+    out.mkdir(parents=True, exist_ok=True)
+    (out / "config.json").write_text(json.dumps(config_to_dict(cfg), indent=1))
+    tensors: Dict[str, torch.Tensor] = {}
+
+    class _Grab(HybridModel):
+        def set_weights(self, get) -> None:          # the generator of random_init, without a model
+            for name in param_shapes(cfg):
+                tensors[name] = get(name).contiguous()
+    _Grab.random_init(cfg, "cpu", seed=seed)
+    save_file(tensors, str(out / "model.safetensors"), metadata={"format": "pt"})
+    return out
+
+
 def load_transformer(path: str, device, tp_rank: int = 0, tp_size: int = 1, comm=None,
                      cfg: Optional[ModelConfig] = None, ep_size: int = 1,
                      ep_mode: str = "allreduce") -> TransformerModel:

@@ -325,3 +325,39 @@ def test_serving_steps_launch_only_the_kernel_library(dtype):
         torch.cuda.synchronize()
     assert all(len(o.token_ids[0]) == 5 for o in outs)
     assert audit.kernels == {}, audit.kernels
+
+
+def test_checkpoint_directory_through_the_registry_and_the_command_line(tmp_path, capsys):
+    """A Nidozen checkpoint directory is found by its config.json, loaded with the checkpoint's
+    tensor names, and answers a question through the command line beside a transformer member."""
+    from llm_consensus_amd import cli
+    from llm_consensus_amd.models.loader import load_model, write_random_hybrid_checkpoint
+    from llm_consensus_amd.models.registry import resolve
+
+    cfg = config_from_dict(config([attn(ff=24), gru(width=24), gla(), attn(kv_from=0, ff=0)], width=32, vocab=300))
+    ck = write_random_hybrid_checkpoint(cfg, str(tmp_path / "nidozen"), seed=3)
+    assert resolve(str(ck)).name == "hybrid"
+    m = load_model(str(ck), "cpu", dtype=torch.float32)
+    assert [L.spec.type for L in m.layers] == ["attention", "mingru", "gla", "attention"] and m.layers[2].spec.rank == 6
+    toml = tmp_path / "e.toml"
+    toml.write_text(f"""strategy = "majority_vote"
+decision_mode = "logprob"
+choices = "ABCD"
+[sampling]
+temperature = 0.0
+max_new_tokens = 4
+[models.h]
+path = "{ck}"
+[models.t]
+preset = "tiny-llama"
+[[members]]
+name = "hybrid"
+model = "h"
+[[members]]
+name = "llama"
+model = "t"
+""")
+    q = tmp_path / "q.txt"
+    q.write_text("Which? A. a B. b C. c D. d\n")
+    assert cli.main(["--config", str(toml), "--questions", str(q), "--device", "cpu", "--no-warm-up"]) == 0
+    assert capsys.readouterr().out.strip()[-1] in "ABCD"
