@@ -9,33 +9,16 @@
 // A step's sequences are described by cu_q [B+1] (row ranges), positions [T] and slots [B]
 // (state slot of the sequence; < 0: padding row of a recorded step, skipped). A sequence whose
 // first row is at position 0 starts from a zero state, so slots are never cleared.
-#include "common.h"
+#include "hybrid_common.h"
 
 namespace {
-
-template <bool F32>
-struct Act;
-template <>
-struct Act<true> {
-  typedef float type;
-  static LC_DEVICE float load(const float* p, size_t i) { return p[i]; }
-  static LC_DEVICE void store(float* p, size_t i, float v) { p[i] = v; }
-};
-template <>
-struct Act<false> {
-  typedef bf16_t type;
-  static LC_DEVICE float load(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }
-  static LC_DEVICE void store(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
-};
-
-LC_DEVICE float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
-LC_DEVICE float siluf_(float x) { return x / (1.f + expf(-x)); }
 
 // ---------------------------------------------------------------- embedding -> fp32 stream (+ activation copy)
 template <bool EF32, bool AF32>
 __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* __restrict__ E, float* __restrict__ x,
                                   void* __restrict__ xa, int T, int d, int vocab, const int32_t* __restrict__ feed_tok,
-                                  const int32_t* __restrict__ feed_rows) {
+                                  const int32_t* __restrict__ feed_rows, float scale,
+                                  const int32_t* __restrict__ positions, const float* __restrict__ inv_freq) {
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= T) return;
@@ -47,8 +30,14 @@ __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* _
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const typename Act<EF32>::type* e = static_cast<const typename Act<EF32>::type*>(E) + static_cast<size_t>(id) * d;
   typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
+  // optional sinusoidal position vector: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i), fp32 angles
+  const float pos = inv_freq != nullptr ? static_cast<float>(positions[row]) : 0.f;
   for (int c = lane; c < d; c += 64) {
-    const float v = Act<EF32>::load(e, c);
+    float v = Act<EF32>::load(e, c) * scale;
+    if (inv_freq != nullptr) {
+      const float ang = pos * inv_freq[c >> 1];
+      v += (c & 1) ? cosf(ang) : sinf(ang);
+    }
     x[static_cast<size_t>(row) * d + c] = v;
     if (a != nullptr) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, v);
   }
@@ -167,8 +156,7 @@ __global__ void gla_prepare_kernel(const float* __restrict__ proj, int ld, const
   const int c = static_cast<int>(i - t * HD);
   const float* row = proj + t * ld;
   const float z = decay[i];
-  // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|))
-  const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
+  const float a = expf(logsigmoidf_(z) * inv_tau);
   prep[i] = make_float4(row[c] * qscale, row[HD + c], a, 0.f);
 }
 
@@ -179,7 +167,8 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
                                                       int D, int Dv, int mode, int nseg, int seg_len,
-                                                      float* __restrict__ cs, float* __restrict__ ca) {
+                                                      float* __restrict__ cs, float* __restrict__ ca,
+                                                      long long state_stride, int ones) {
   const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
@@ -190,7 +179,8 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   if (r0 >= q1) return;
   const bool live = dv < Dv;
   float S[DMAX];
-  float* st = state + (static_cast<size_t>(slot) * H + h) * D * Dv;
+  float* st = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * D * Dv;
+  const int Dvr = Dv - ones;                      // value columns that come from the projection
   float* seg_s = cs != nullptr ? cs + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D * Dv : nullptr;
   const float* from = mode == 2 ? seg_s : st;
   const bool zero = mode == 1 || (mode == 0 && positions[q0] == 0);
@@ -213,7 +203,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
       const int d = threadIdx.x + 64 * i;
       dst[i] = d < D ? x[d] : make_float4(0.f, 0.f, 1.f, 0.f);
     }
-    vv = live ? proj[static_cast<size_t>(t) * ld + 2 * H * D + h * Dv + dv] : 0.f;
+    vv = !live ? 0.f : (dv < Dvr ? proj[static_cast<size_t>(t) * ld + 2 * H * D + h * Dvr + dv] : 1.f);
   };
   fetch(r0, nxt, vnxt);
   for (int t = r0; t < r1; ++t) {
@@ -262,7 +252,8 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
 // segment STARTS from on exit (the sequence's own state for s = 0). One thread per state element.
 __global__ void gla_carry_kernel(float* __restrict__ cs, const float* __restrict__ ca, const float* __restrict__ state,
                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                 const int32_t* __restrict__ slots, int H, int D, int Dv, int nseg, int seg_len) {
+                                 const int32_t* __restrict__ slots, int H, int D, int Dv, int nseg, int seg_len,
+                                 long long state_stride) {
   const int b = blockIdx.y;
   const size_t n = static_cast<size_t>(H) * D * Dv;
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -270,7 +261,7 @@ __global__ void gla_carry_kernel(float* __restrict__ cs, const float* __restrict
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
   if (i >= n || slot < 0 || q1 <= q0) return;
   const size_t hd = i / Dv;                         // (head, key channel)
-  float carry = positions[q0] == 0 ? 0.f : state[static_cast<size_t>(slot) * n + i];
+  float carry = positions[q0] == 0 ? 0.f : state[static_cast<size_t>(slot) * state_stride + i];
   const int used = (q1 - q0 + seg_len - 1) / seg_len;
   for (int s = 0; s < used; ++s) {
     float* p = cs + (static_cast<size_t>(b) * nseg + s) * n + i;
@@ -280,24 +271,161 @@ __global__ void gla_carry_kernel(float* __restrict__ cs, const float* __restrict
   }
 }
 
-// Per head: o / sqrt(mean(o^2) + eps) * w, times silu(gate). One wave per (row, head).
+// Per head: o / sqrt(mean(o^2) + eps) * w, times act(gate). One wave per (row, head). Heads are
+// ``ld_head`` apart in o (>= Dv); head h reads the weights w[h * w_stride ...] (w_stride 0: one
+// weight vector for all heads); act is silu (gate_kind 0) or sigmoid (1). With ``m`` [T, H] the
+// read-out is first divided by max(|o[Dv]|, exp(-m)) + 1e-6, o[Dv] being the column behind the head's values
+// (a matrix memory's normaliser . q, m its running maximum).
 template <bool AF32>
 __global__ void headnorm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                      const float* __restrict__ gate, int ld_gate, void* __restrict__ out, int T, int H,
-                                     int Dv, float eps) {
+                                     int Dv, float eps, int ld_head, int w_stride, int gate_kind,
+                                     const float* __restrict__ m) {
   const int idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (idx >= T * H) return;
   const int row = idx / H, h = idx % H;
-  const float* orow = o + static_cast<size_t>(row) * H * Dv + h * Dv;
+  const float* orow = o + (static_cast<size_t>(row) * H + h) * ld_head;
   const float* grow = gate + static_cast<size_t>(row) * ld_gate + h * Dv;
+  const float* wh = w + static_cast<size_t>(h) * w_stride;
+  float inv = 1.f;
+  if (m != nullptr) inv = 1.f / (fmaxf(fabsf(orow[Dv]), expf(-m[idx])) + 1e-6f);
   float ss = 0.f;
-  for (int c = lane; c < Dv; c += 64) ss += orow[c] * orow[c];
+  for (int c = lane; c < Dv; c += 64) {
+    const float v = orow[c] * inv;
+    ss += v * v;
+  }
   ss = wave_sum(ss);
-  const float r = 1.f / sqrtf(ss / static_cast<float>(Dv) + eps);
+  const float r = inv / sqrtf(ss / static_cast<float>(Dv) + eps);
   typename Act<AF32>::type* dst = static_cast<typename Act<AF32>::type*>(out);
-  for (int c = lane; c < Dv; c += 64)
-    Act<AF32>::store(dst, static_cast<size_t>(row) * H * Dv + h * Dv + c, orow[c] * r * w[c] * siluf_(grow[c]));
+  for (int c = lane; c < Dv; c += 64) {
+    const float g = grow[c];
+    Act<AF32>::store(dst, static_cast<size_t>(row) * H * Dv + h * Dv + c,
+                     orow[c] * r * wh[c] * (gate_kind == 0 ? siluf_(g) : sigmoidf_(g)));
+  }
+}
+
+// ---------------------------------------------------------------- mLSTM: gates and prepared operands
+// proj [T, ld]: q | k | v | output gate | input-gate logits [H] | forget-gate logits [H]. Per head, with
+// i = cap tanh(. / cap) and f = log sigmoid(cap tanh(. / cap)) (cap 0: no cap), the running maximum
+// m_t = max(f_t + m_(t-1), i_t) (0 before the first token) stabilises
+//   S_t = a_t S_(t-1) + b_t k_t v_t^T,  a_t = exp(f_t + m_(t-1) - m_t),  b_t = exp(i_t - m_t).
+// One wave per (head, sequence): 64 tokens at a time, the lanes compute the gates of their tokens and
+// the maxima come from a wave scan (m -> max(m + F, I) composes as (F1 + F2, max(I1 + F2, I2))).
+// Writes (a, b) per (token, head), m per (token, head), and the sequence's last m behind its state.
+LC_DEVICE float soft_cap(float x, float cap) { return cap > 0.f ? cap * tanhf(x / cap) : x; }
+
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(const float* __restrict__ proj, int ld, int col_i,
+                                                         float* __restrict__ state, long long state_stride,
+                                                         long long m_offset, const int32_t* __restrict__ cu_q,
+                                                         const int32_t* __restrict__ positions,
+                                                         const int32_t* __restrict__ slots, float2* __restrict__ gates,
+                                                         float* __restrict__ m_out, int H, float cap) {
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const int slot = slots[b];
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (slot < 0 || q1 <= q0) return;
+  float* ms = state + static_cast<size_t>(slot) * state_stride + m_offset + h;
+  float m = positions[q0] == 0 ? 0.f : *ms;
+  for (int r0 = q0; r0 < q1; r0 += 64) {
+    const int t = r0 + lane;
+    const bool valid = t < q1;
+    const float iv = valid ? soft_cap(proj[static_cast<size_t>(t) * ld + col_i + h], cap) : -INFINITY;
+    const float fv = valid ? logsigmoidf_(soft_cap(proj[static_cast<size_t>(t) * ld + col_i + H + h], cap)) : 0.f;
+    float F = fv, I = iv;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float Fp = __shfl_up(F, off, 64), Ip = __shfl_up(I, off, 64);
+      if (lane >= off) {
+        I = fmaxf(Ip + F, I);
+        F = Fp + F;
+      }
+    }
+    const float mt = fmaxf(m + F, I);
+    float mp = __shfl_up(mt, 1, 64);
+    if (lane == 0) mp = m;
+    if (valid) {
+      gates[static_cast<size_t>(t) * H + h] = make_float2(expf(fv + mp - mt), expf(iv - mt));
+      m_out[static_cast<size_t>(t) * H + h] = mt;
+    }
+    m = __shfl(mt, min(63, q1 - 1 - r0), 64);
+  }
+  if (lane == 0) *ms = m;
+}
+
+// (q / sqrt(D), b k, a, -) per (token, head, key channel): the operands of the scan below.
+__global__ void mlstm_prepare_kernel(const float* __restrict__ proj, int ld, const float2* __restrict__ gates,
+                                     float4* __restrict__ prep, long long n, int H, int D, float qscale) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int HD = H * D;
+  const long long t = i / HD;
+  const int c = static_cast<int>(i - t * HD);
+  const float* row = proj + t * ld;
+  const float2 g = gates[t * H + c / D];
+  prep[i] = make_float4(row[c] * qscale, row[HD + c] * g.y, g.x, 0.f);
+}
+
+// ---------------------------------------------------------------- pre-norm residual step
+// x += y (when y is given), xa = x * rsqrt(mean(x^2) + eps) * w (when w is given). WAVES as in the
+// scalar-gain kernel above.
+template <bool AF32, int WAVES>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                          const float* __restrict__ w, float eps,
+                                                          void* __restrict__ xa, int T, int d) {
+  __shared__ float red[16];
+  constexpr int LANES = 64 * WAVES;
+  const int row = WAVES == 1 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  const int lane = WAVES == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  if (WAVES == 1 && row >= T) return;
+  float* xr = x + static_cast<size_t>(row) * d;
+  const float* yr = y != nullptr ? y + static_cast<size_t>(row) * d : nullptr;
+  float ss = 0.f;
+  for (int c = lane; c < d; c += LANES) {
+    float v = xr[c];
+    if (yr != nullptr) {
+      v += yr[c];
+      xr[c] = v;
+    }
+    ss += v * v;
+  }
+  if (w == nullptr) return;                         // the same for every thread
+  ss = WAVES == 1 ? wave_sum(ss) : block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / static_cast<float>(d) + eps);
+  typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
+  for (int c = lane; c < d; c += LANES) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, xr[c] * r * w[c]);
+}
+
+// act(gate) * up of y [T, 2n] = (gate | up); act: relu (kind 0) or silu (1).
+template <bool AF32>
+__global__ void glu_kernel(const float* __restrict__ y, void* __restrict__ out, long long total, int n, int kind) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long t = i / n;
+  const int c = static_cast<int>(i - t * n);
+  const float g = y[t * 2 * n + c], u = y[t * 2 * n + n + c];
+  Act<AF32>::store(static_cast<typename Act<AF32>::type*>(out), i, (kind == 0 ? fmaxf(g, 0.f) : siluf_(g)) * u);
+}
+
+// ---------------------------------------------------------------- latent attention: the cached row
+// One wave per token: c = rms_norm(proj[t, col0 : col0 + R]) * w goes to cache [blocks, 1, BS, R] at the
+// token's slot.
+template <bool CF32>
+__global__ void latent_write_kernel(const float* __restrict__ proj, int ld, int col0, int R, const float* __restrict__ w,
+                                    float eps, const int32_t* __restrict__ slot_mapping, void* __restrict__ cache,
+                                    int BS, int T) {
+  const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t >= T) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const float* row = proj + static_cast<size_t>(t) * ld + col0;
+  float ss = 0.f;
+  for (int c = lane; c < R; c += 64) ss += row[c] * row[c];
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / static_cast<float>(R) + eps);
+  typename Act<CF32>::type* dst = static_cast<typename Act<CF32>::type*>(cache);
+  for (int c = lane; c < R; c += 64) Act<CF32>::store(dst, static_cast<size_t>(slot) * R + c, row[c] * r * w[c]);
 }
 
 // ---------------------------------------------------------------- attention: norms, rotation, cache write
@@ -718,18 +846,73 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ 
   }
 }
 
+// ---------------------------------------------------------------- per-head products
+// C[m, h, :] = W[h] A[m, h, :] for H heads side by side: A [M, H*K] (row stride lda), W [H, N, K],
+// C [M, H*N]. The tiling of gemm_any_kernel with the head as the third grid dimension. With
+// ``gate`` [M, H] (row stride ld_gate) the head's outputs are scaled by sigmoid(gate[m, h]).
+template <bool AF32, bool WF32, bool CF32>
+__global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict__ A, int lda, const void* __restrict__ W,
+                                                          void* __restrict__ C, const float* __restrict__ gate,
+                                                          int ld_gate, int M, int H, int N, int K) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  const int h = blockIdx.z;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A) + static_cast<size_t>(h) * K;
+  const typename Act<WF32>::type* w = static_cast<const typename Act<WF32>::type*>(W) + static_cast<size_t>(h) * N * K;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    for (int i = threadIdx.x; i < 64 * 16; i += 256) {
+      const int r = i >> 4, k = i & 15;
+      As[k][r] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * lda + k0 + k) : 0.f;
+      Ws[k][r] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        av[i] = As[k][ty * 4 + i];
+        wv[i] = Ws[k][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * wv[j];
+    }
+    __syncthreads();
+  }
+  typename Act<CF32>::type* c = static_cast<typename Act<CF32>::type*>(C);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = m0 + ty * 4 + i;
+    if (r >= M) continue;
+    const float g = gate != nullptr ? sigmoidf_(gate[static_cast<size_t>(r) * ld_gate + h]) : 1.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + tx * 4 + j;
+      if (col < N) Act<CF32>::store(c, (static_cast<size_t>(r) * H + h) * N + col, acc[i][j] * g);
+    }
+  }
+}
+
 }  // namespace
 
 // ================================================================= launchers
 LC_EXPORT int lc_embed_rows(const void* ids, const void* E, int e_f32, void* x, void* xa, int act_f32, int T, int d,
-                            int vocab, const void* feed_tok, const void* feed_rows, hipStream_t st) {
+                            int vocab, const void* feed_tok, const void* feed_rows, float scale, const void* positions,
+                            const void* inv_freq, hipStream_t st) {
   if (T <= 0) return 0;
-  if (d <= 0 || vocab <= 0) return -1;
+  if (d <= 0 || vocab <= 0 || (inv_freq != nullptr && (positions == nullptr || (d & 1)))) return -1;
   const dim3 grid((T + 3) / 4), block(256);
 #define LC_EMB(E32, A32)                                                                                      \
   embed_rows_kernel<E32, A32><<<grid, block, 0, st>>>(static_cast<const int32_t*>(ids), E, static_cast<float*>(x), \
                                                       xa, T, d, vocab, static_cast<const int32_t*>(feed_tok), \
-                                                      static_cast<const int32_t*>(feed_rows))
+                                                      static_cast<const int32_t*>(feed_rows), scale,          \
+                                                      static_cast<const int32_t*>(positions),                 \
+                                                      static_cast<const float*>(inv_freq))
   if (e_f32 && act_f32) LC_EMB(true, true);
   else if (e_f32) LC_EMB(true, false);
   else if (act_f32) LC_EMB(false, true);
@@ -800,20 +983,15 @@ LC_EXPORT int lc_mingru_scan(const void* zxg, void* state, const void* cu_q, con
   LC_RETURN_LAST_ERROR();
 }
 
-// ``prep``: T * H * D float4 of scratch for the per-token operands (gla_prepare_kernel).
-LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* state, const void* cu_q,
-                          const void* positions, const void* slots, void* out, int T, int B, int H, int D, int Dv,
-                          float tau, int max_len, void* scratch, void* prep, hipStream_t st) {
-  if (B <= 0) return 0;
-  if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + H * Dv || !(tau > 0.f)) return -1;
+// The scan over prepared operands (``prep``: T * H * D float4, see the prepare kernels): per head
+// S <- a S + k v^T over Dv value columns, the last ``ones`` of which read v = 1.
+static int launch_linear_scan(const void* proj, int ld, const void* prep, void* state, long long state_stride,
+                              const void* cu_q, const void* positions, const void* slots, void* out, int B, int H, int D,
+                              int Dv, int ones, int max_len, void* scratch, hipStream_t st) {
   const bool segmented = max_len > 2 * kScanSegment;
-  if (prep == nullptr || T <= 0 || (segmented && scratch == nullptr)) return -1;
+  if (segmented && scratch == nullptr) return -1;
   const int nseg = segmented ? (max_len + kScanSegment - 1) / kScanSegment : 1;
   const dim3 grid((Dv + 63) / 64, H, B * nseg), block(64);
-  const long long n = static_cast<long long>(T) * H * D;
-  gla_prepare_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st>>>(
-      static_cast<const float*>(proj), ld, static_cast<const float*>(decay), static_cast<float4*>(prep), n, H * D,
-      1.f / tau, 1.f / sqrtf(static_cast<float>(D)));
   float* cs = static_cast<float*>(scratch);
   float* ca = segmented ? cs + static_cast<size_t>(B) * nseg * H * D * Dv : nullptr;
 #define LC_GLA(DMAX, MODE)                                                                                             \
@@ -821,7 +999,7 @@ LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* sta
                                                 static_cast<float*>(state), static_cast<const int32_t*>(cu_q),      \
                                                 static_cast<const int32_t*>(positions),                             \
                                                 static_cast<const int32_t*>(slots), static_cast<float*>(out), H, D, \
-                                                Dv, MODE, nseg, kScanSegment, cs, ca)
+                                                Dv, MODE, nseg, kScanSegment, cs, ca, state_stride, ones)
 #define LC_GLA_D(MODE)          \
   if (D <= 32) LC_GLA(32, MODE);  \
   else if (D <= 64) LC_GLA(64, MODE); \
@@ -832,7 +1010,8 @@ LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* sta
     const size_t n = static_cast<size_t>(H) * D * Dv;
     gla_carry_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256), B), dim3(256), 0, st>>>(
         cs, ca, static_cast<const float*>(state), static_cast<const int32_t*>(cu_q),
-        static_cast<const int32_t*>(positions), static_cast<const int32_t*>(slots), H, D, Dv, nseg, kScanSegment);
+        static_cast<const int32_t*>(positions), static_cast<const int32_t*>(slots), H, D, Dv, nseg, kScanSegment,
+        state_stride);
     LC_GLA_D(2);
   } else {
     LC_GLA_D(0);
@@ -842,17 +1021,122 @@ LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* sta
   LC_RETURN_LAST_ERROR();
 }
 
-LC_EXPORT int lc_headnorm_gate(const void* o, const void* w, const void* gate, int ld_gate, void* out, int act_f32,
-                               int T, int H, int Dv, float eps, hipStream_t st) {
+// ``prep``: T * H * D float4 of scratch for the per-token operands (gla_prepare_kernel).
+LC_EXPORT int lc_gla_scan(const void* proj, int ld, const void* decay, void* state, long long state_stride,
+                          const void* cu_q, const void* positions, const void* slots, void* out, int T, int B, int H,
+                          int D, int Dv, float tau, int max_len, void* scratch, void* prep, hipStream_t st) {
+  if (B <= 0) return 0;
+  if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + H * Dv || !(tau > 0.f)) return -1;
+  if (prep == nullptr || T <= 0 || state_stride < static_cast<long long>(H) * D * Dv) return -1;
+  const long long n = static_cast<long long>(T) * H * D;
+  gla_prepare_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st>>>(
+      static_cast<const float*>(proj), ld, static_cast<const float*>(decay), static_cast<float4*>(prep), n, H * D,
+      1.f / tau, 1.f / sqrtf(static_cast<float>(D)));
+  return launch_linear_scan(proj, ld, prep, state, state_stride, cu_q, positions, slots, out, B, H, D, Dv, 0, max_len,
+                            scratch, st);
+}
+
+// mLSTM: gates and running maxima, prepared operands, then the scan over Dv + 1 value columns (the
+// extra column, v = 1, is the normaliser). ``prep``: T * H * (4 D + 2) floats; ``out`` [T, H * (Dv + 1)];
+// ``m_out`` [T, H]; a slot of ``state`` holds H * D * (Dv + 1) floats and then the H maxima.
+LC_EXPORT int lc_mlstm_scan(const void* proj, int ld, void* state, long long state_stride, const void* cu_q,
+                            const void* positions, const void* slots, void* out, void* m_out, int T, int B, int H, int D,
+                            int Dv, float cap, int max_len, void* scratch, void* prep, hipStream_t st) {
+  if (B <= 0 || T <= 0) return 0;
+  if (H <= 0 || D <= 0 || Dv <= 0 || D > 256 || ld < 2 * H * D + 2 * H * Dv + 2 * H || cap < 0.f) return -1;
+  const long long n_s = static_cast<long long>(H) * D * (Dv + 1);
+  if (prep == nullptr || m_out == nullptr || state_stride < n_s + H) return -1;
+  const long long n = static_cast<long long>(T) * H * D;
+  float2* gates = reinterpret_cast<float2*>(static_cast<float4*>(prep) + n);
+  mlstm_gates_kernel<<<dim3(H, B), dim3(64), 0, st>>>(
+      static_cast<const float*>(proj), ld, 2 * H * D + 2 * H * Dv, static_cast<float*>(state), state_stride, n_s,
+      static_cast<const int32_t*>(cu_q), static_cast<const int32_t*>(positions), static_cast<const int32_t*>(slots), gates,
+      static_cast<float*>(m_out), H, cap);
+  mlstm_prepare_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st>>>(
+      static_cast<const float*>(proj), ld, gates, static_cast<float4*>(prep), n, H, D, 1.f / sqrtf(static_cast<float>(D)));
+  return launch_linear_scan(proj, ld, prep, state, state_stride, cu_q, positions, slots, out, B, H, D, Dv + 1, 1, max_len,
+                            scratch, st);
+}
+
+LC_EXPORT int lc_add_rmsnorm(void* x, const void* y, const void* w, float eps, void* xa, int act_f32, int T, int d,
+                             hipStream_t st) {
   if (T <= 0) return 0;
-  if (H <= 0 || Dv <= 0 || ld_gate < H * Dv) return -1;
+  if (d <= 0 || (w != nullptr && xa == nullptr)) return -1;
+  const bool few = T <= 512;
+  const dim3 grid(few ? T : (T + 3) / 4), block(256);
+#define LC_AN(A32, WAVES)                                                                                          \
+  add_rmsnorm_kernel<A32, WAVES><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y),    \
+                                                         static_cast<const float*>(w), eps, xa, T, d)
+  if (act_f32 && few) LC_AN(true, 4);
+  else if (act_f32) LC_AN(true, 1);
+  else if (few) LC_AN(false, 4);
+  else LC_AN(false, 1);
+#undef LC_AN
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_glu(const void* y, void* out, int act_f32, int T, int n, int kind, hipStream_t st) {
+  if (T <= 0 || n <= 0) return 0;
+  const long long total = static_cast<long long>(T) * n;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
+  if (act_f32) glu_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, total, n, kind);
+  else glu_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, total, n, kind);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_latent_write(const void* proj, int ld, int col0, int R, const void* w, float eps, const void* slot_mapping,
+                              void* cache, int cache_f32, int BS, int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (R <= 0 || col0 < 0 || ld < col0 + R || BS <= 0) return -1;
+  const dim3 grid((T + 3) / 4), block(256);
+  if (cache_f32)
+    latent_write_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, col0, R,
+                                                      static_cast<const float*>(w), eps,
+                                                      static_cast<const int32_t*>(slot_mapping), cache, BS, T);
+  else
+    latent_write_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(proj), ld, col0, R,
+                                                       static_cast<const float*>(w), eps,
+                                                       static_cast<const int32_t*>(slot_mapping), cache, BS, T);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_head_linear(const void* A, int a_f32, int lda, const void* W, int w_f32, void* C, int c_f32,
+                             const void* gate, int ld_gate, int M, int H, int N, int K, hipStream_t st) {
+  if (M <= 0 || N <= 0 || H <= 0) return 0;
+  if (K <= 0 || lda < H * K || H > 65535 || (gate != nullptr && ld_gate < H)) return -1;
+  const dim3 grid((N + 63) / 64, (M + 63) / 64, H), block(256);
+#define LC_HL(A32, W32, C32)                                                                                   \
+  head_linear_kernel<A32, W32, C32><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, M, H, \
+                                                            N, K)
+  const int sel = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
+  switch (sel) {
+    case 0: LC_HL(false, false, false); break;
+    case 1: LC_HL(false, false, true); break;
+    case 2: LC_HL(false, true, false); break;
+    case 3: LC_HL(false, true, true); break;
+    case 4: LC_HL(true, false, false); break;
+    case 5: LC_HL(true, false, true); break;
+    case 6: LC_HL(true, true, false); break;
+    default: LC_HL(true, true, true); break;
+  }
+#undef LC_HL
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_headnorm_gate(const void* o, const void* w, const void* gate, int ld_gate, void* out, int act_f32,
+                               int T, int H, int Dv, float eps, int ld_head, int w_stride, int gate_kind, const void* m,
+                               hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || Dv <= 0 || ld_gate < H * Dv || ld_head < Dv || (m != nullptr && ld_head < Dv + 1)) return -1;
   const dim3 grid((T * H + 3) / 4), block(256);
   if (act_f32)
     headnorm_gate_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(o), static_cast<const float*>(w),
-                                                       static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps);
+                                                       static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps,
+                                                       ld_head, w_stride, gate_kind, static_cast<const float*>(m));
   else
     headnorm_gate_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(o), static_cast<const float*>(w),
-                                                        static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps);
+                                                        static_cast<const float*>(gate), ld_gate, out, T, H, Dv, eps,
+                                                        ld_head, w_stride, gate_kind, static_cast<const float*>(m));
   LC_RETURN_LAST_ERROR();
 }
 

@@ -1,8 +1,32 @@
 """Hybrid decoders: a stack whose layers each pick one mixer -- chunk-masked attention over the
-paged cache, minGRU, or gated linear attention -- around an fp32 residual stream.
+paged cache, latent attention over a cache of compressed rows, minGRU, gated linear attention or
+mLSTM -- around an fp32 residual stream.
 
-The design served here is Nidozen. Its ``config.json`` lists the layers (``layers[i].type``,
-``.mixer`` sizes, ``.mlp``), and every size and constant comes from there or from a tensor's shape:
+Two designs are served, told apart by ``architecture`` in ``config.json`` (``DESIGNS``); the file lists
+the layers (``layers[i].type``, ``.mixer`` sizes, ``.mlp``), and every size and constant comes from
+there or from a tensor's shape.
+
+Telurax (pre-norm):
+
+* ``x = embed[token] * embedding.scale`` plus a sinusoidal position vector (entry 2i: sin, 2i+1: cos of
+  ``p * 10000^(-2i/width)``); a layer computes ``x += mixer(n1(x))`` and, if it has a feed-forward,
+  ``x += ff(n2(x))`` with ``n(x) = x / sqrt(mean(x^2) + eps) * (1 + w)``; logits are
+  ``head . n_final(x) * logit_scale``;
+* ``latent_attention``: queries ``W_q h`` per head; ONE compressed row per token, the RMS-normed
+  ``W_dkv h`` (plain weight), is cached, and every head's keys and values are linear maps of it
+  (``W_uk``, ``W_uv``). The maps are moved to the query and to the output side (scores
+  ``(W_uk_h^T q_h) . c_j``, output ``W_uv_h sum_j p_j c_j``), so attention runs over the cached rows
+  themselves: H query heads, one key/value head of the latent's width, causal softmax, no positions.
+  Each head's output is scaled by ``sigmoid(W_g h)_h`` before ``W_o``;
+* ``mlstm``: per head a matrix memory ``S <- a S + b k v^T`` with a normaliser ``n <- a n + b k``,
+  ``a = exp(f + m' - m)``, ``b = exp(i - m)``, ``m = max(f + m', i)`` (m' the previous maximum, 0 at
+  the start), soft-capped gate logits; read out ``S^T q / (max(|n.q|, exp(-m)) + 1e-6)``, unit RMS
+  per head, a weight over all heads, an output gate ``sigmoid(W_g h)``, ``W_o``;
+* feed-forwards: ``down(relu(gate h) * up h)``, or a routed mixture (softmax router, bias-corrected
+  group-limited top-k choice, identity experts that return their input, a shared expert; experts are
+  ``down(relu(up h)^2)``).
+
+Nidozen (norms on the sublayer outputs):
 
 * a layer computes ``x += norm1(mixer(x))`` and, if it has a feed-forward, ``x += norm2(ff(x))``:
   the sublayers read the stream itself and the norm (RMS with ONE gain for all coordinates) sits
@@ -35,7 +59,47 @@ import torch
 from .. import ops
 
 ARCHITECTURE = "Nidozen"
-MIXERS = ("attention", "mingru", "gla")
+
+
+@dataclass(frozen=True)
+class Design:
+    """What a design fixes for all of its models."""
+
+    name: str
+    mixers: Tuple[str, ...]
+    pre_norm: bool = False          # norms with a weight per coordinate on the sublayer INPUTS (else: one-gain norms on the outputs)
+    norm_offset: float = 0.0        # stored norm weights are offsets from this value
+    pos_base: float = 0.0           # > 0: a sinusoidal position vector of this base is added to the embedding
+    dense_ff: str = "relu2"         # dense feed-forward: down(relu(up x)^2) | "glu_relu": down(relu(gate x) * up x)
+
+
+DESIGNS: Dict[str, Design] = {
+    "Nidozen": Design("Nidozen", ("attention", "mingru", "gla")),
+    "Telurax": Design("Telurax", ("latent_attention", "mlstm"), pre_norm=True, norm_offset=1.0, pos_base=10000.0,
+                      dense_ff="glu_relu"),
+}
+MIXERS = tuple(m for d in DESIGNS.values() for m in d.mixers)
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """A routed feed-forward: ``experts`` small relu^2 feed-forwards of width ``ff`` plus ``identity``
+    experts without tensors; the router's ``experts + identity`` outputs form ``groups`` equal runs of
+    neighbours of which the ``keep`` best stay eligible; ``top`` are chosen per token, weighted by their
+    softmax score times ``scale``; ``shared_ff`` > 0: a shared expert of that width runs for every token."""
+
+    experts: int
+    ff: int
+    top: int
+    identity: int = 0
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
+
+    @property
+    def outputs(self) -> int:
+        return self.experts + self.identity
 
 
 @dataclass(frozen=True)
@@ -57,12 +121,21 @@ class LayerSpec:
     rank: int = 0                # width of the decay's low-rank bottleneck (from the tensor's shape)
     # mingru
     width: int = 0
-    # feed-forward (0: none)
+    # latent attention: width of the cached compressed row
+    kv_rank: int = 0
+    # mlstm: soft cap of the gate logits (0: none)
+    gate_cap: float = 0.0
+    # feed-forward (0: none); ``moe``: a routed one instead of the dense one
     ff: int = 0
+    moe: Optional[MoESpec] = None
 
     @property
     def owns_kv(self) -> bool:
         return self.type == "attention" and self.kv_from < 0
+
+    @property
+    def has_ff(self) -> bool:
+        return self.ff > 0 or self.moe is not None
 
     def state_size(self) -> int:
         """fp32 numbers of recurrent state per sequence."""
@@ -70,7 +143,15 @@ class LayerSpec:
             return self.width
         if self.type == "gla":
             return self.heads * self.dim * self.vdim
+        if self.type == "mlstm":          # S with the normaliser as an extra column, then the running maxima
+            return self.heads * self.dim * (self.vdim + 1) + self.heads
         return 0
+
+    def cache_elems(self) -> int:
+        """Cached elements per token."""
+        if self.owns_kv:
+            return self.kv_heads * (self.dim + self.vdim)
+        return self.kv_rank if self.type == "latent_attention" else 0
 
 
 @dataclass(frozen=True)
@@ -83,6 +164,12 @@ class HybridConfig:
     max_position: int = 1 << 20
     model_type: str = "nidozen"
     architecture: str = ARCHITECTURE
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+
+    @property
+    def design(self) -> Design:
+        return DESIGNS[self.architecture]
 
     @property
     def num_layers(self) -> int:
@@ -94,14 +181,14 @@ class HybridConfig:
 
     @property
     def num_heads(self) -> int:
-        return max([l.heads for l in self.layers if l.type == "attention"] or [1])
+        return max([l.heads for l in self.layers if l.type in ("attention", "latent_attention")] or [1])
 
     @property
     def num_kv_heads(self) -> int:
         return max([l.kv_heads for l in self.layers if l.type == "attention"] or [1])
 
     def kv_elems_per_token(self) -> int:
-        return sum(l.kv_heads * (l.dim + l.vdim) for l in self.layers if l.owns_kv)
+        return sum(l.cache_elems() for l in self.layers)
 
     def kv_bytes_per_token(self, bytes_per_elem: int = 2) -> int:
         return self.kv_elems_per_token() * bytes_per_elem
@@ -118,9 +205,27 @@ class HybridConfig:
     def validate(self) -> None:
         if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
             raise ValueError(f"{self.name}: vocab, width and at least one layer are needed")
+        if self.architecture not in DESIGNS:
+            raise ValueError(f"{self.name}: unknown design {self.architecture!r} (known: {', '.join(DESIGNS)})")
+        known = self.design.mixers
+        if self.design.pos_base > 0 and self.hidden_size % 2:
+            raise ValueError(f"{self.name}: a sinusoidal position vector needs an even width")
         for i, l in enumerate(self.layers):
-            if l.type not in MIXERS:
-                raise ValueError(f"{self.name}: layer {i}: unknown mixer {l.type!r} (known: {', '.join(MIXERS)})")
+            if l.type not in known:
+                raise ValueError(f"{self.name}: layer {i}: unknown mixer {l.type!r} (known: {', '.join(known)})")
+            if l.type in ("latent_attention", "mlstm") and (l.heads <= 0 or l.dim <= 0 or l.vdim <= 0):
+                raise ValueError(f"{self.name}: layer {i}: heads, dim and vdim are needed")
+            if l.type == "latent_attention" and (l.kv_rank <= 0 or l.kv_rank > 256):
+                raise ValueError(f"{self.name}: layer {i}: the attention kernels take a latent width of 1..256")
+            if l.type == "mlstm" and (l.dim > 256 or l.gate_cap < 0):
+                raise ValueError(f"{self.name}: layer {i}: mLSTM takes dim <= 256 and a gate cap >= 0")
+            if l.moe is not None:
+                m = l.moe
+                if m.experts <= 0 or m.ff <= 0 or m.identity < 0 or m.top <= 0 or m.groups <= 0 or m.outputs % m.groups:
+                    raise ValueError(f"{self.name}: layer {i}: experts, their width and `top` are needed, and the groups "
+                                     f"must divide experts + identity")
+                if not 1 <= m.keep <= m.groups or m.top > m.keep * (m.outputs // m.groups) or m.top > 32:
+                    raise ValueError(f"{self.name}: layer {i}: the kept groups must hold `top` (at most 32) router outputs")
             if l.type == "mingru" and l.width <= 0:
                 raise ValueError(f"{self.name}: layer {i}: minGRU needs a width")
             if l.type in ("attention", "gla") and (l.heads <= 0 or l.dim <= 0 or l.vdim <= 0):
@@ -150,20 +255,35 @@ def _numel(shape) -> int:
     return n
 
 
-def config_from_dict(c: dict, name: str = "nidozen", tensor_shapes: Optional[Dict[str, tuple]] = None) -> HybridConfig:
-    """Parses a Nidozen ``config.json``. ``tensor_shapes`` (name -> shape of the checkpoint's
+def _mlp_of(name: str, i: int, mlp: Optional[dict], design: Design):
+    """(ff, MoESpec or None) of a layer's ``mlp`` entry."""
+    if mlp is None:
+        return 0, None
+    kind = mlp.get("kind", "dense")
+    if kind == "dense":
+        return int(mlp["ff"]), None
+    if kind != "moe" or not design.pre_norm:
+        raise ValueError(f"{name}: layer {i}: feed-forward kind {kind!r} is not supported")
+    r, g = mlp["router"], mlp["router"].get("groups") or {}
+    shared = mlp.get("shared") or {}
+    return 0, MoESpec(experts=int(r["experts"]), ff=int(mlp["expert"]["ff"]), top=int(r["top"]),
+                      identity=int(r.get("identity", 0)), groups=int(g.get("count", 1)), keep=int(g.get("keep", g.get("count", 1))),
+                      scale=float(r.get("scale", 1.0)), shared_ff=int(shared.get("ff", 0)))
+
+
+def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict[str, tuple]] = None) -> HybridConfig:
+    """Parses the ``config.json`` of a hybrid design. ``tensor_shapes`` (name -> shape of the checkpoint's
     tensors) supplies the sizes the configuration leaves to the tensors."""
-    if c.get("architecture") != ARCHITECTURE:
-        raise ValueError(f"{name}: architecture {c.get('architecture')!r} is not {ARCHITECTURE}")
+    arch = c.get("architecture")
+    if arch not in DESIGNS:
+        raise ValueError(f"{name}: architecture {arch!r} is not one of {', '.join(DESIGNS)}")
+    design = DESIGNS[arch]
     layers = []
     for i, L in enumerate(c["layers"]):
         t, m = L["type"], L.get("mixer") or {}
-        mlp = L.get("mlp")
-        ff = 0
-        if mlp is not None:
-            if mlp.get("kind", "dense") != "dense":
-                raise ValueError(f"{name}: layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported")
-            ff = int(mlp["ff"])
+        if t not in design.mixers:
+            raise ValueError(f"{name}: layer {i}: unknown mixer {t!r} (known: {', '.join(design.mixers)})")
+        ff, moe = _mlp_of(name, i, L.get("mlp"), design)
         if t == "attention":
             mask, rot = m.get("mask") or {}, m.get("rot") or {}
             kvf = m.get("kv_from")
@@ -180,11 +300,18 @@ def config_from_dict(c: dict, name: str = "nidozen", tensor_shapes: Optional[Dic
                 rank = int(tensor_shapes[f"l{i}.mix.a1"][0])
             layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
                                     tau=float(m["tau"]), rank=rank or 16, ff=ff))
+        elif t == "latent_attention":
+            layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                    kv_rank=int(m["kv_rank"]), scale=float(m.get("scale", int(m["dim"]) ** -0.5)),
+                                    ff=ff, moe=moe))
         else:
-            raise ValueError(f"{name}: layer {i}: unknown mixer {t!r} (known: {', '.join(MIXERS)})")
+            layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                    gate_cap=float(m.get("gate_cap", 0.0)), ff=ff, moe=moe))
     cfg = HybridConfig(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
                        rms_eps=float(c["norm"]["eps"]), layers=tuple(layers),
-                       max_position=int(c.get("max_position", 1 << 20)))
+                       max_position=int(c.get("max_position", 1 << 20)), model_type=arch.lower(), architecture=arch,
+                       embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                       logit_scale=float(c.get("logit_scale", 1.0)))
     cfg.validate()
     return cfg
 
@@ -200,11 +327,26 @@ def config_to_dict(cfg: HybridConfig) -> dict:
                 m["kv_from"] = l.kv_from
         elif l.type == "mingru":
             m = {"width": l.width}
-        else:
+        elif l.type == "gla":
             m = {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "tau": l.tau, "rank": l.rank}
-        layers.append({"type": l.type, "mixer": m, "mlp": {"kind": "dense", "ff": l.ff} if l.ff else None})
-    return {"architecture": ARCHITECTURE, "vocab": cfg.vocab_size, "width": cfg.hidden_size,
-            "norm": {"eps": cfg.rms_eps}, "layers": layers}
+        elif l.type == "latent_attention":
+            m = {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "kv_rank": l.kv_rank, "scale": l.scale}
+        else:
+            m = {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "gate_cap": l.gate_cap}
+        mlp = {"kind": "dense", "ff": l.ff} if l.ff else None
+        if l.moe is not None:
+            e = l.moe
+            mlp = {"kind": "moe", "expert": {"ff": e.ff},
+                   "router": {"experts": e.experts, "identity": e.identity, "top": e.top, "scale": e.scale,
+                              "groups": {"count": e.groups, "keep": e.keep}},
+                   "shared": {"ff": e.shared_ff} if e.shared_ff else None}
+        layers.append({"type": l.type, "mixer": m, "mlp": mlp})
+    out = {"architecture": cfg.architecture, "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+           "norm": {"eps": cfg.rms_eps}, "layers": layers}
+    if cfg.design.pre_norm:
+        out["embedding"] = {"scale": cfg.embed_scale}
+        out["logit_scale"] = cfg.logit_scale
+    return out
 
 
 def config_from_path(path: str) -> HybridConfig:
@@ -224,12 +366,13 @@ def config_from_path(path: str) -> HybridConfig:
 def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
     """Checkpoint tensor names -> shapes (linear weights are [out, in])."""
     d = cfg.hidden_size
+    norm = (d,) if cfg.design.pre_norm else ()
     out: Dict[str, tuple] = {"embed": (cfg.vocab_size, d)}
     for i, l in enumerate(cfg.layers):
         p = f"l{i}."
-        out[p + "norm1"] = ()
-        if l.ff:
-            out[p + "norm2"] = ()
+        out[p + "norm1"] = norm
+        if l.has_ff:
+            out[p + "norm2"] = norm
         m = p + "mix."
         if l.type == "attention":
             out[m + "q"], out[m + "q.b"], out[m + "q.norm"] = (l.heads * l.dim, d), (l.heads * l.dim,), (l.heads * l.dim,)
@@ -243,15 +386,37 @@ def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
                 out[m + n] = (l.width, d)
             out[m + "z.b"], out[m + "x.b"] = (l.width,), (l.width,)
             out[m + "o"] = (d, l.width)
-        else:
+        elif l.type == "gla":
             out[m + "q"], out[m + "k"] = (l.heads * l.dim, d), (l.heads * l.dim, d)
             out[m + "v"], out[m + "g"] = (l.heads * l.vdim, d), (l.heads * l.vdim, d)
             out[m + "a1"], out[m + "a2"], out[m + "a2.b"] = (l.rank, d), (l.heads * l.dim, l.rank), (l.heads * l.dim,)
             out[m + "norm"] = (l.vdim,)
             out[m + "o"] = (d, l.heads * l.vdim)
-        if l.ff:
-            out[p + "mlp.up"], out[p + "mlp.down"] = (l.ff, d), (d, l.ff)
-    out["final.norm"] = ()
+        elif l.type == "latent_attention":
+            out[m + "q"] = (l.heads * l.dim, d)
+            out[m + "dkv"], out[m + "dkv.norm"] = (l.kv_rank, d), (l.kv_rank,)
+            out[m + "uk"], out[m + "uv"] = (l.heads * l.dim, l.kv_rank), (l.heads * l.vdim, l.kv_rank)
+            out[m + "g"] = (l.heads, d)
+            out[m + "o"] = (d, l.heads * l.vdim)
+        else:
+            out[m + "q"], out[m + "k"] = (l.heads * l.dim, d), (l.heads * l.dim, d)
+            out[m + "v"], out[m + "g"] = (l.heads * l.vdim, d), (l.heads * l.vdim, d)
+            out[m + "o"], out[m + "norm"] = (d, l.heads * l.vdim), (l.heads * l.vdim,)
+            for n in ("i", "f"):
+                out[m + n], out[m + n + ".b"] = (l.heads, d), (l.heads,)
+        f = p + "mlp."
+        if l.moe is not None:
+            e = l.moe
+            for j in range(e.experts):
+                out[f + f"e{j}.up"], out[f + f"e{j}.down"] = (e.ff, d), (d, e.ff)
+            out[f + "router"], out[f + "correction"] = (e.outputs, d), (e.outputs,)
+            if e.shared_ff:
+                out[f + "shared.up"], out[f + "shared.down"] = (e.shared_ff, d), (d, e.shared_ff)
+        elif l.ff:
+            if cfg.design.dense_ff == "glu_relu":
+                out[f + "gate"] = (l.ff, d)
+            out[f + "up"], out[f + "down"] = (l.ff, d), (d, l.ff)
+    out["final.norm"] = norm
     out["head"] = (cfg.vocab_size, d)
     return out
 
@@ -268,9 +433,11 @@ class StepLayout:
 
 
 class HybridCache:
-    """Paged keys / values of the attention layers that own any, and the fp32 state slots of the
-    recurrent layers, in ONE pool. Key planes are [blocks, G, BS, dim], value planes
-    [blocks, G, BS, vdim] in the model's activation type; a state plane is [slots, size] fp32."""
+    """Paged keys / values of the attention layers that own any, the paged compressed rows of the
+    latent-attention layers, and the fp32 state slots of the recurrent layers, in ONE pool. Key
+    planes are [blocks, G, BS, dim], value planes [blocks, G, BS, vdim], latent planes
+    [blocks, 1, BS, kv_rank] (keys and values at once) in the model's activation type; a state
+    plane is [slots, size] fp32."""
 
     def __init__(self, cfg: HybridConfig, num_blocks: int, block_size: int, num_slots: int, device,
                  dtype: torch.dtype, alloc=None):
@@ -287,6 +454,8 @@ class HybridCache:
             if l.owns_kv:
                 plan.append(("k", i, take(num_blocks * l.kv_heads * block_size * l.dim * es)))
                 plan.append(("v", i, take(num_blocks * l.kv_heads * block_size * l.vdim * es)))
+            elif l.type == "latent_attention":
+                plan.append(("c", i, take(num_blocks * block_size * l.kv_rank * es)))
             elif l.state_size():
                 plan.append(("s", i, take(max(1, num_slots) * l.state_size() * 4)))
         total = max(off, 256)
@@ -307,6 +476,9 @@ class HybridCache:
             elif kind == "v":
                 n = num_blocks * l.kv_heads * block_size * l.vdim * es
                 self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.vdim)
+            elif kind == "c":
+                n = num_blocks * block_size * l.kv_rank * es
+                self._k[i] = self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, 1, block_size, l.kv_rank)
             else:
                 n = max(1, num_slots) * l.state_size() * 4
                 self._s[i] = raw[at:at + n].view(torch.float32).view(max(1, num_slots), l.state_size())
@@ -343,11 +515,21 @@ class HybridLayer:
     k_norm: Optional[torch.Tensor] = None
     inv_freq: Optional[torch.Tensor] = None         # fp32 [rot_dims/2]
     decay_up: Optional[ops.LinearWeight] = None     # gla: bottleneck -> decay logits
-    head_norm: Optional[torch.Tensor] = None        # gla: fp32 [vdim]
+    head_norm: Optional[torch.Tensor] = None        # gla: fp32 [vdim]; mlstm: fp32 [H*vdim]
+    gate_up: Optional[ops.LinearWeight] = None      # gated dense feed-forward: gate | up
+    latent_norm: Optional[torch.Tensor] = None      # latent attention: fp32 [kv_rank]
+    key_up_t: Optional[torch.Tensor] = None         # latent attention: [H, kv_rank, dim], head h's key map transposed
+    value_up: Optional[torch.Tensor] = None         # latent attention: [H, vdim, kv_rank]
+    router: Optional[ops.LinearWeight] = None       # routed feed-forward: [experts + identity, d]
+    correction: Optional[torch.Tensor] = None       # fp32 [experts + identity]
+    experts_up: Optional[torch.Tensor] = None       # [E, ff, d]
+    experts_down: Optional[torch.Tensor] = None     # [E, d, ff]
+    shared_up: Optional[ops.LinearWeight] = None
+    shared_down: Optional[ops.LinearWeight] = None
 
 
 class HybridModel:
-    """One Nidozen model on one device. Same surface as ``TransformerModel`` towards the engine:
+    """One model of a hybrid design on one device. Same surface as ``TransformerModel`` towards the engine:
     ``forward`` (the residual stream of the step's rows), ``logits``, ``make_cache``."""
 
     tp_rank, tp_size, ep_size, comm = 0, 1, 1, None
@@ -367,6 +549,11 @@ class HybridModel:
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self._max_len = 1
         self._portions = (0, 0)
+        self.pos_freq: Optional[torch.Tensor] = None    # fp32 [d/2]: frequencies of the sinusoidal position vector
+        if cfg.design.pos_base > 0:
+            half = cfg.hidden_size // 2
+            f = torch.tensor([cfg.design.pos_base ** (-2.0 * j / cfg.hidden_size) for j in range(half)], dtype=torch.float64)
+            self.pos_freq = f.to(torch.float32).to(self.device)
 
     # ------------------------------------------------------------------ construction
     def set_weights(self, get) -> None:
@@ -388,8 +575,13 @@ class HybridModel:
 
         def f32(t: torch.Tensor) -> torch.Tensor:
             return t.to(torch.float32).reshape(-1).contiguous()
+
+        def norm_w(name: str, scale: float = 1.0) -> torch.Tensor:
+            # stored as an offset from the design's base value; the kernels multiply by the sum
+            return ((f32(load(name)) + c.design.norm_offset) * scale).contiguous()
         self.embed = load("embed").to(dt).contiguous()
-        self.final_norm = f32(load("final.norm"))
+        # the logits' scale rides on the final norm's weight
+        self.final_norm = norm_w("final.norm", c.logit_scale) if c.design.pre_norm else f32(load("final.norm"))
         self.lm_head = lin(load("head"))
         self.layers = []
         for i, l in enumerate(c.layers):
@@ -411,16 +603,50 @@ class HybridModel:
                 bias = torch.cat([load(m + "z.b"), load(m + "x.b"), torch.zeros(l.width, device=dev)])
                 proj = lin(torch.cat([load(m + "z"), load(m + "x"), load(m + "g")], 0), bias)
                 out = lin(load(m + "o"))
-            else:
+            elif l.type == "gla":
                 proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "a1")], 0))
                 # the bottleneck's output is an fp32 column slice of the fused projection: the small
                 # second product takes it as it is through the shape-agnostic kernel
                 kw["decay_up"] = ops.LinearWeight.from_dense(load(m + "a2"), load(m + "a2.b"), dev, dtype=dt, plain=True)
                 kw["head_norm"] = f32(load(m + "norm"))
                 out = lin(load(m + "o"))
-            if l.ff:
-                kw.update(norm2=f32(load(p + "norm2")), up=lin(load(p + "mlp.up")), down=lin(load(p + "mlp.down")))
-            self.layers.append(HybridLayer(l, f32(load(p + "norm1")), proj, out, **kw))
+            elif l.type == "latent_attention":
+                # queries | compressed row | one gate logit per head, in one product
+                proj = lin(torch.cat([load(m + n) for n in ("q", "dkv", "g")], 0))
+                kw["latent_norm"] = f32(load(m + "dkv.norm"))
+                kw["key_up_t"] = load(m + "uk").view(l.heads, l.dim, l.kv_rank).transpose(1, 2).to(dt).contiguous()
+                kw["value_up"] = load(m + "uv").view(l.heads, l.vdim, l.kv_rank).to(dt).contiguous()
+                out = lin(load(m + "o"))
+            else:
+                hd, hv = l.heads * l.dim, l.heads * l.vdim
+                bias = torch.cat([torch.zeros(2 * hd + 2 * hv, device=dev), load(m + "i.b"), load(m + "f.b")])
+                proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "i", "f")], 0), bias)
+                kw["head_norm"] = f32(load(m + "norm"))
+                out = lin(load(m + "o"))
+            f = p + "mlp."
+            if l.moe is not None:
+                e = l.moe
+                kw["router"] = ops.LinearWeight.from_dense(load(f + "router"), None, dev, dtype=dt, plain=True)
+                kw["correction"] = f32(load(f + "correction"))
+                kw["experts_up"] = torch.stack([load(f + f"e{j}.up") for j in range(e.experts)]).to(dt).contiguous()
+                kw["experts_down"] = torch.stack([load(f + f"e{j}.down") for j in range(e.experts)]).to(dt).contiguous()
+                if e.shared_ff:
+                    kw.update(shared_up=lin(load(f + "shared.up")), shared_down=lin(load(f + "shared.down")))
+            elif l.ff:
+                if c.design.dense_ff == "glu_relu":
+                    kw["gate_up"] = lin(torch.cat([load(f + "gate"), load(f + "up")], 0))
+                else:
+                    kw["up"] = lin(load(f + "up"))
+                kw["down"] = lin(load(f + "down"))
+            if c.design.pre_norm:
+                n1 = norm_w(p + "norm1")
+                if l.has_ff:
+                    kw["norm2"] = norm_w(p + "norm2")
+            else:
+                n1 = f32(load(p + "norm1"))
+                if l.has_ff:
+                    kw["norm2"] = f32(load(p + "norm2"))
+            self.layers.append(HybridLayer(l, n1, proj, out, **kw))
 
     @classmethod
     def random_init(cls, cfg: HybridConfig, device, seed: int = 0, dtype: torch.dtype = torch.bfloat16,
@@ -434,12 +660,18 @@ class HybridModel:
         def get(name: str) -> torch.Tensor:
             shape = shapes[name]
             gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFFFFFFFFFF)
+            offset_norm = cfg.design.norm_offset != 0.0 and name.split(".")[-1] in ("norm1", "norm2") or \
+                (cfg.design.norm_offset != 0.0 and name == "final.norm")
             if len(shape) == 2:
                 t = torch.randn(shape, generator=gen) * (1.0 if name == "embed" else shape[1] ** -0.5)
+            elif offset_norm:
+                t = 0.1 * torch.randn(shape, generator=gen)
             elif name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
                 t = 1.0 + 0.1 * torch.randn(shape, generator=gen)
-            elif name.endswith("a2.b"):
+            elif name.endswith("a2.b") or name.endswith("mix.f.b"):
                 t = 2.0 + torch.randn(shape, generator=gen)
+            elif name.endswith("correction"):
+                t = 0.02 * torch.randn(shape, generator=gen)
             else:
                 t = 0.1 * torch.randn(shape, generator=gen)
             return t.to(torch.bfloat16)
@@ -449,8 +681,10 @@ class HybridModel:
     def weight_bytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size() + self.lm_head.nbytes()
         for L in self.layers:
-            for w in (L.proj, L.out, L.up, L.down, L.decay_up):
+            for w in (L.proj, L.out, L.up, L.down, L.decay_up, L.gate_up, L.router, L.shared_up, L.shared_down):
                 n += w.nbytes() if w is not None else 0
+            for t in (L.key_up_t, L.value_up, L.experts_up, L.experts_down):
+                n += t.numel() * t.element_size() if t is not None else 0
         return n
 
     # ------------------------------------------------------------------ engine surface
@@ -490,6 +724,8 @@ class HybridModel:
         T = token_ids.numel()
         self._portions = (meta.block_tables.shape[0], meta.prefill_tokens if meta.riders is not None else T) \
             if meta.is_prefill else (0, 0)
+        if c.design.pre_norm:
+            return self._forward_pre_norm(token_ids, positions, slot_mapping, meta, lay, cache, taps)
         x, xa = ops.embed_rows(token_ids, self.embed, dt, meta.token_feed)
         for i, L in enumerate(self.layers):
             l = L.spec
@@ -503,14 +739,80 @@ class HybridModel:
                 y = self._gla(i, L, xa, positions, lay, cache)
             xa = ops.scalar_norm_add(x, y, L.norm1, eps, dt)
             if L.up is not None:
-                if L.up.is_packed or not x.is_cuda:
-                    u = ops.relu2(ops.linear(xa, L.up, out_f32=True), dt)
-                else:
-                    u = ops.linear_any(xa, L.up, out_f32=dt == torch.float32, epi_relu2=True)
-                xa = ops.scalar_norm_add(x, ops.linear(u, L.down, out_f32=True), L.norm2, eps, dt)
+                xa = ops.scalar_norm_add(x, ops.linear(self._relu2_up(xa, L.up), L.down, out_f32=True), L.norm2, eps, dt)
             if taps is not None:
                 taps.append(x.clone())
         return x
+
+    def _relu2_up(self, xa: torch.Tensor, up: ops.LinearWeight) -> torch.Tensor:
+        """relu(up x)^2 in the activation type: an epilogue of the shape-agnostic product, one more
+        launch behind the packed MFMA product."""
+        if up.is_packed or not xa.is_cuda:
+            return ops.relu2(ops.linear(xa, up, out_f32=True), self.dtype)
+        return ops.linear_any(xa, up, out_f32=self.dtype == torch.float32, epi_relu2=True)
+
+    def _forward_pre_norm(self, token_ids, positions, slot_mapping, meta, lay: StepLayout, cache: HybridCache,
+                          taps: Optional[list]) -> torch.Tensor:
+        """Layers whose sublayers read the normed stream: every residual sum and the norm that feeds
+        the next sublayer are one launch (``ops.add_rmsnorm``)."""
+        c, dt, eps = self.cfg, self.dtype, self.cfg.rms_eps
+        x, _ = ops.embed_rows(token_ids, self.embed, None, meta.token_feed, c.embed_scale, positions, self.pos_freq)
+        xa = ops.add_rmsnorm(x, None, self.layers[0].norm1, eps, dt)
+        for i, L in enumerate(self.layers):
+            l = L.spec
+            if l.type == "latent_attention":
+                y = self._latent_attention(i, L, xa, positions, slot_mapping, lay, cache)
+            else:
+                y = self._mlstm(i, L, xa, positions, lay, cache)
+            nxt = self.layers[i + 1].norm1 if i + 1 < len(self.layers) else None
+            if l.has_ff:
+                xa = ops.add_rmsnorm(x, y, L.norm2, eps, dt)
+                y = self._routed_ff(L, xa) if l.moe is not None else self._dense_ff(L, xa)
+            xa = ops.add_rmsnorm(x, y, nxt, eps, dt)
+            if taps is not None:
+                taps.append(x.clone())
+        return x
+
+    def _dense_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
+        if L.gate_up is not None:
+            return ops.linear(ops.glu(ops.linear(xa, L.gate_up, out_f32=True), self.dtype, "relu"), L.down, out_f32=True)
+        return ops.linear(self._relu2_up(xa, L.up), L.down, out_f32=True)
+
+    def _routed_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
+        e = L.spec.moe
+        z = ops.linear_any(xa, L.router, out_f32=True)
+        ids, wts = ops.route_grouped(z, L.correction, e.top, e.groups, e.keep, e.scale)
+        offsets, sorted_src, slot_of = ops.moe_sort(ids, e.outputs)
+        rows = ids.numel()
+        act = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, self.dtype, rows, relu2_epi=True)
+        ye = ops.grouped_linear(act, None, offsets, L.experts_down, torch.float32, rows)
+        shared = None
+        if L.shared_up is not None:
+            shared = ops.linear(self._relu2_up(xa, L.shared_up), L.shared_down, out_f32=True)
+        return ops.moe_mix(ye, slot_of, ids, wts, xa, e.experts, shared)
+
+    def _latent_attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
+        l = L.spec
+        hd, R = l.heads * l.dim, l.kv_rank
+        proj = ops.linear(xa, L.proj, out_f32=True)                 # q | compressed row | gate logits
+        cc = cache.k(i)
+        ops.latent_write(proj, hd, L.latent_norm, self.cfg.rms_eps, slot_mapping, cc)
+        q = ops.head_linear(proj[:, :hd], L.key_up_t, torch.float32)        # queries in the latent's coordinates
+        a = ops.attn_masked(q, cc, cc, lay.block_tables, lay.cu_q, lay.row_seq, positions, l.heads, 1, R, R, l.scale,
+                            0, 0, self.dtype, n_portions=self._portions[0], portion_rows=self._portions[1],
+                            max_len=self._max_len)
+        o = ops.head_linear(a, L.value_up, self.dtype, gate=proj[:, hd + R:hd + R + l.heads])
+        return ops.linear(o, L.out, out_f32=True)
+
+    def _mlstm(self, i: int, L: HybridLayer, xa, positions, lay: StepLayout, cache: HybridCache):
+        l = L.spec
+        hd, hv = l.heads * l.dim, l.heads * l.vdim
+        proj = ops.linear(xa, L.proj, out_f32=True)                 # q | k | v | gate | input gate | forget gate
+        o, m = ops.mlstm_scan(proj, cache.state(i), lay.cu_q, positions, lay.state_slots, l.heads, l.dim, l.vdim,
+                              l.gate_cap, self._max_len)
+        y = ops.mlstm_out(o, m, L.head_norm, proj[:, 2 * hd + hv:2 * hd + 2 * hv], l.heads, l.vdim, self.cfg.rms_eps,
+                          self.dtype)
+        return ops.linear(y, L.out, out_f32=True)
 
     def _attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
         l = L.spec
@@ -537,7 +839,10 @@ class HybridModel:
 
     def logits(self, hidden_rows: torch.Tensor) -> torch.Tensor:
         """fp32 logits [R, V] of the given rows of the residual stream (final norm, then the head)."""
-        xa = ops.scalar_norm_add(hidden_rows, None, self.final_norm, self.cfg.rms_eps, self.dtype)
+        if self.cfg.design.pre_norm:
+            xa = ops.add_rmsnorm(hidden_rows.contiguous(), None, self.final_norm, self.cfg.rms_eps, self.dtype)
+        else:
+            xa = ops.scalar_norm_add(hidden_rows, None, self.final_norm, self.cfg.rms_eps, self.dtype)
         return ops.linear(xa, self.lm_head, out_f32=True)
 
     def target_logprobs(self, hidden_rows: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:

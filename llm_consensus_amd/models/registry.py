@@ -2,7 +2,7 @@
 
 A checkpoint names its family in ``config.json``: Hugging Face checkpoints by ``model_type``
 (llama, qwen2, mistral, mixtral -> ``TransformerModel``), hybrid decoders by ``architecture``
-(Nidozen -> ``HybridModel``). ``resolve(path)`` returns the family entry; ``loader.load_model``
+(Nidozen, Telurax -> ``HybridModel``). ``resolve(path)`` returns the family entry; ``loader.load_model``
 and ``loader.build_model`` go through it, so the engine, the back ends and the command-line
 tools take either kind of directory.
 """
@@ -21,6 +21,10 @@ class Family:
     load: Callable[..., object]                   # (path, device, **kw) -> model with weights
     kernel_groups: Tuple[str, ...]                # source groups of the kernel library it needs (build_native.py)
 
+
+# the designs models/hybrid.py serves (its ``DESIGNS``), named here so that finding a checkpoint's
+# family does not import the model code
+HYBRID_DESIGNS = ("Nidozen", "Telurax")
 
 _FAMILIES: Dict[str, Family] = {}
 _BY_KEY: Dict[Tuple[str, str], str] = {}          # (config key, value) -> family name
@@ -68,7 +72,8 @@ def _register_builtin() -> None:
 
     register(Family("transformer", tcfg.from_hf_config, load_transformer, ("base", "transformer")),
              [("model_type", t) for t in tcfg.SUPPORTED_MODEL_TYPES])
-    register(Family("hybrid", hybrid_config, load_hybrid, ("base", "hybrid")), [("architecture", "Nidozen")])
+    register(Family("hybrid", hybrid_config, load_hybrid, ("base", "hybrid")),
+             [("architecture", a) for a in HYBRID_DESIGNS])
 
 
 _register_builtin()

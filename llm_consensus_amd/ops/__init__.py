@@ -902,22 +902,31 @@ def linear_any(x: torch.Tensor, w: LinearWeight, out_f32: bool = True, epi_relu2
 
 
 def embed_rows(ids: torch.Tensor, E: torch.Tensor, act_dtype: Optional[torch.dtype],
-               feed: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
-    """Rows E[ids] as (fp32 [T, d], copy in ``act_dtype`` or None). E is bf16 or fp32; with
-    ``act_dtype`` fp32 the copy IS the fp32 tensor. ``feed`` as in ``embed``. Also the row gather
-    of an fp32 matrix."""
+               feed: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, scale: float = 1.0,
+               positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None):
+    """Rows E[ids] * scale as (fp32 [T, d], copy in ``act_dtype`` or None). E is bf16 or fp32; with
+    ``act_dtype`` fp32 the copy IS the fp32 tensor. ``feed`` as in ``embed``. With ``positions`` and
+    ``inv_freq`` (fp32 [d/2]) a sinusoidal position vector is added: entry 2i is sin(p f_i), entry
+    2i + 1 cos(p f_i), angles in fp32. Also the row gather of an fp32 matrix."""
     T, d = ids.numel(), E.shape[1]
+    if inv_freq is not None and (positions is None or 2 * inv_freq.numel() != d):
+        raise ValueError("embed_rows: the position table needs positions and d / 2 frequencies")
     if not ids.is_cuda:
         if feed is not None:
             tok, rows = feed
             ids = torch.where(rows >= 0, tok[rows.clamp_min(0).long()].to(ids.dtype), ids)
         x = ref.embed(ids, E).float()
+        if scale != 1.0:
+            x = x * scale
+        if inv_freq is not None:
+            x = x + ref.sinusoid_rows(positions, inv_freq)
         return x, (x if act_dtype in (None, torch.float32) else x.to(act_dtype))
     x = torch.empty(T, d, dtype=torch.float32, device=E.device)
     xa = torch.empty(T, d, dtype=act_dtype, device=E.device) if act_dtype == torch.bfloat16 else None
     _hip().call("lc_embed_rows", ids.data_ptr(), E.data_ptr(), _f32flag(E.dtype), x.data_ptr(), _hip().ptr(xa), 0, T, d,
                 E.shape[0], feed[0].data_ptr() if feed is not None else None,
-                feed[1].data_ptr() if feed is not None else None)
+                feed[1].data_ptr() if feed is not None else None, float(scale),
+                positions.data_ptr() if inv_freq is not None else None, _hip().ptr(inv_freq))
     return x, (xa if xa is not None else (x if act_dtype is not None else None))
 
 
@@ -996,7 +1005,7 @@ def gla_scan(proj: torch.Tensor, decay_logits: torch.Tensor, state: torch.Tensor
     scratch = _scan_scratch(B, max_len, H * D * Dv, H * D, proj.device)
     prep = torch.empty(T * H * D * 4, dtype=torch.float32, device=proj.device)     # (q, k, decay, -) per channel
     _hip().call("lc_gla_scan", proj.data_ptr(), proj.stride(0), decay_logits.data_ptr(), state.data_ptr(),
-                cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), T, B, H, D, Dv,
+                state.stride(0), cu_q.data_ptr(), positions.data_ptr(), slots.data_ptr(), out.data_ptr(), T, B, H, D, Dv,
                 float(tau), int(max_len), _hip().ptr(scratch), prep.data_ptr())
     return out
 
@@ -1013,7 +1022,7 @@ def headnorm_gate(o: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, Dv: int,
     o = o.contiguous()
     out = torch.empty(T, n, dtype=act_dtype, device=o.device)
     _hip().call("lc_headnorm_gate", o.data_ptr(), w.data_ptr(), gate.data_ptr(), gate.stride(0), out.data_ptr(),
-                _f32flag(act_dtype), T, n // Dv, Dv, float(eps))
+                _f32flag(act_dtype), T, n // Dv, Dv, float(eps), Dv, 0, 0, None)
     return out
 
 
@@ -1090,4 +1099,173 @@ def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
         _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
                     block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
                     out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window))
+    return out
+
+
+# ---- pre-norm designs, latent attention, mLSTM, routed feed-forwards (hybrid.hip, hybrid_moe.hip) ----
+def add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float,
+                act_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """The residual step of a pre-norm layer in one launch: x (fp32 stream, in place) += y, and the
+    input of the next sublayer x / sqrt(mean(x^2) + eps) * w in ``act_dtype`` (``w``: fp32 [d], any
+    offset already folded in). Without ``y`` only the norm; without ``w`` only the sum (returns None)."""
+    if not x.is_cuda:
+        return ref.add_rmsnorm(x, y, w, eps, act_dtype)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("add_rmsnorm: the residual stream is a contiguous fp32 tensor")
+    if y is not None and (y.shape != x.shape or y.dtype != torch.float32):
+        raise ValueError("add_rmsnorm: the sublayer output must be fp32 of the stream's shape")
+    if y is None and w is None:
+        return None
+    xa = torch.empty(T, d, dtype=act_dtype, device=x.device) if w is not None else None
+    _hip().call("lc_add_rmsnorm", x.data_ptr(), _hip().ptr(y.contiguous() if y is not None else None), _hip().ptr(w),
+                float(eps), _hip().ptr(xa), _f32flag(act_dtype), T, d)
+    return xa
+
+
+def latent_write(proj: torch.Tensor, col0: int, w: torch.Tensor, eps: float, slot_mapping: torch.Tensor,
+                 cache: torch.Tensor) -> None:
+    """The compressed key/value row of every token: rms_norm(proj[:, col0:col0 + R]) * w, written to
+    ``cache`` [blocks, 1, BS, R] at the rows' slots (rows with slot < 0 are skipped)."""
+    if not proj.is_cuda:
+        return ref.latent_write(proj, col0, w, eps, slot_mapping, cache)
+    R = cache.shape[3]
+    if proj.dtype != torch.float32 or proj.stride(1) != 1 or cache.shape[1] != 1 or col0 + R > proj.shape[1]:
+        raise ValueError("latent_write: fp32 projections and a one-head cache plane of the latent's width")
+    _hip().call("lc_latent_write", proj.data_ptr(), proj.stride(0), int(col0), R, w.data_ptr(), float(eps),
+                slot_mapping.data_ptr(), cache.data_ptr(), _f32flag(cache.dtype), cache.shape[2], proj.shape[0])
+
+
+def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per-head products y[t, h] = W[h] x[t, h]: x [T, H*K] (may be a column slice), W [H, N, K]
+    row-major, y [T, H*N] in ``out_dtype``; fp32 accumulation. ``gate`` [T, H] (logits, may be a
+    column slice): y[t, h] *= sigmoid(gate[t, h])."""
+    if not x.is_cuda:
+        return ref.head_linear(x, W, out_dtype, gate)
+    H, N, K = W.shape
+    M = x.shape[0]
+    if x.shape[1] != H * K or x.stride(1) != 1 or not W.is_contiguous():
+        raise ValueError("head_linear: activations [T, H*K] against weights [H, N, K]")
+    if gate is not None and (gate.shape != (M, H) or gate.dtype != torch.float32 or gate.stride(1) != 1):
+        raise ValueError("head_linear: the gate is an fp32 [T, H] matrix")
+    y = torch.empty(M, H * N, dtype=out_dtype, device=x.device)
+    _hip().call("lc_head_linear", x.data_ptr(), _f32flag(x.dtype), max(x.stride(0), H * K), W.data_ptr(), _f32flag(W.dtype),
+                y.data_ptr(), _f32flag(out_dtype), _hip().ptr(gate), max(gate.stride(0), H) if gate is not None else 0,
+                M, H, N, K)
+    return y
+
+
+def mlstm_scan(proj: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor,
+               slots: torch.Tensor, H: int, D: int, Dv: int, cap: float, max_len: int = 1):
+    """mLSTM matrix memory over the step's sequences. proj fp32 [T, >= 2HD + 2HDv + 2H] holds
+    q | k | v | output gate | input-gate logits | forget-gate logits; state fp32
+    [slots, H*D*(Dv+1) + H] (per head S with the normaliser as an extra column, then the running
+    maxima; updated in place). Gates are soft-capped (``cap`` > 0). Returns (read-out fp32
+    [T, H*(Dv+1)], last column per head = normaliser . q; running maximum fp32 [T, H])."""
+    if not proj.is_cuda:
+        return ref.mlstm_scan(proj, state, cu_q, positions, slots, H, D, Dv, cap)
+    T = proj.shape[0]
+    need = 2 * H * D + 2 * H * Dv + 2 * H
+    if proj.dtype != torch.float32 or state.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] < need:
+        raise ValueError("mlstm_scan: fp32 projections q | k | v | g | i | f and fp32 state")
+    if state.shape[1] != H * D * (Dv + 1) + H or D > 256:
+        raise ValueError("mlstm_scan: the state does not fit the head sizes (key width at most 256)")
+    B = slots.numel()
+    Da = Dv + 1
+    out = torch.empty(T, H * Da, dtype=torch.float32, device=proj.device)
+    m = torch.empty(T, H, dtype=torch.float32, device=proj.device)
+    prep = torch.empty(T * H * (4 * D + 2), dtype=torch.float32, device=proj.device)    # operands, then (a, b) per (token, head)
+    scratch = _scan_scratch(B, max_len, H * D * Da, H * D, proj.device)
+    _hip().call("lc_mlstm_scan", proj.data_ptr(), proj.stride(0), state.data_ptr(), state.stride(0), cu_q.data_ptr(),
+                positions.data_ptr(), slots.data_ptr(), out.data_ptr(), m.data_ptr(), T, B, H, D, Dv, float(cap),
+                int(max_len), _hip().ptr(scratch), prep.data_ptr())
+    return out, m
+
+
+def mlstm_out(o: torch.Tensor, m: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, H: int, Dv: int, eps: float,
+              act_dtype: torch.dtype) -> torch.Tensor:
+    """From ``mlstm_scan``'s read-out: per head o[:Dv] / (max(|o[Dv]|, exp(-m)) + 1e-6), scaled to
+    unit RMS, times w [H*Dv], times sigmoid(gate) (fp32 [T, H*Dv], may be a column slice)."""
+    if not o.is_cuda:
+        return ref.mlstm_out(o, m, w, gate, H, Dv, eps, act_dtype)
+    T = o.shape[0]
+    if o.shape[1] != H * (Dv + 1) or gate.shape != (T, H * Dv) or gate.stride(1) != 1 or w.numel() != H * Dv:
+        raise ValueError("mlstm_out: shapes do not fit the head sizes")
+    out = torch.empty(T, H * Dv, dtype=act_dtype, device=o.device)
+    _hip().call("lc_headnorm_gate", o.data_ptr(), w.data_ptr(), gate.data_ptr(), gate.stride(0), out.data_ptr(),
+                _f32flag(act_dtype), T, H, Dv, float(eps), Dv + 1, Dv, 1, m.data_ptr())
+    return out
+
+
+def glu(y: torch.Tensor, act_dtype: torch.dtype, kind: str = "relu") -> torch.Tensor:
+    """fp32 y [T, 2n] = (gate | up) -> act(gate) * up [T, n] in ``act_dtype`` (act: relu or silu)."""
+    if not y.is_cuda:
+        return ref.glu(y, act_dtype, kind)
+    T, n = y.shape[0], y.shape[1] // 2
+    y = y.contiguous()
+    out = torch.empty(T, n, dtype=act_dtype, device=y.device)
+    _hip().call("lc_glu", y.data_ptr(), out.data_ptr(), _f32flag(act_dtype), T, n, {"relu": 0, "silu": 1}[kind])
+    return out
+
+
+def route_grouped(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
+    """Group-limited top-k routing over fp32 router logits z [T, n] (see ops.reference.route_grouped):
+    (ids int32 [T, top], weights fp32 [T, top])."""
+    T, n = z.shape
+    if groups < 1 or n % groups or not 1 <= keep <= groups or top > keep * (n // groups):
+        raise ValueError("route_grouped: groups must divide the router's width and the kept groups hold `top` outputs")
+    if not z.is_cuda:
+        return ref.route_grouped(z, correction, top, groups, keep, scale)
+    z = z.contiguous()
+    ids = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    _hip().call("lc_route_grouped", z.data_ptr(), correction.data_ptr(), T, n, top, groups, keep, float(scale),
+                ids.data_ptr(), wts.data_ptr())
+    return ids, wts
+
+
+def moe_sort(ids: torch.Tensor, n: int):
+    """``moe_permute`` for any number of experts (one block, counting sort): (offsets int32 [n+1],
+    sorted_src int32 [T*k], slot_of int32 [T*k])."""
+    if not ids.is_cuda:
+        return moe_permute(ids, n)
+    T, topk = ids.shape
+    dev = ids.device
+    offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    sorted_src = torch.empty(T * topk, dtype=torch.int32, device=dev)
+    slot_of = torch.empty(T * topk, dtype=torch.int32, device=dev)
+    _hip().call("lc_moe_sort", ids.data_ptr(), T, topk, n, offsets.data_ptr(), sorted_src.data_ptr(), slot_of.data_ptr())
+    return offsets, sorted_src, slot_of
+
+
+def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: torch.Tensor, W: torch.Tensor,
+                   out_dtype: torch.dtype, rows: int, relu2_epi: bool = False) -> torch.Tensor:
+    """Per-expert products over expert-sorted rows: position p in [offsets[e], offsets[e+1]) gives
+    W[e] x[row_index[p]] (x[p] without an index). W [E, N, K] row-major of any shape and type, fp32
+    accumulation; ``relu2_epi``: square of relu. Positions of experts >= E are left unwritten."""
+    if not x.is_cuda:
+        return ref.grouped_linear(x, row_index, offsets, W, out_dtype, rows, relu2_epi)
+    E, N, K = W.shape
+    if x.shape[1] != K or x.stride(1) != 1 or not W.is_contiguous():
+        raise ValueError("grouped_linear: activations of the experts' depth")
+    y = torch.empty(rows, N, dtype=out_dtype, device=x.device)
+    _hip().call("lc_gemm_any_grouped", x.data_ptr(), _f32flag(x.dtype), max(x.stride(0), K), _hip().ptr(row_index),
+                offsets.data_ptr(), W.data_ptr(), _f32flag(W.dtype), y.data_ptr(), _f32flag(out_dtype), int(rows), E, N, K,
+                1 if relu2_epi else 0)
+    return y
+
+
+def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, h: torch.Tensor, E: int,
+            shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 [T, d] = sum_k wts[t, k] * (ye[slot_of[t, k]] if ids[t, k] < E else h[t]) (+ shared[t]):
+    experts with ids >= E are identity experts, whose output is the feed-forward's input itself."""
+    if not ye.is_cuda:
+        return ref.moe_mix(ye, slot_of, ids, wts, h, E, shared)
+    T, top = ids.shape
+    d = h.shape[1]
+    if ye.dtype != torch.float32 or (shared is not None and shared.dtype != torch.float32):
+        raise ValueError("moe_mix: fp32 expert outputs")
+    out = torch.empty(T, d, dtype=torch.float32, device=h.device)
+    _hip().call("lc_moe_mix", ye.data_ptr(), slot_of.data_ptr(), ids.data_ptr(), wts.data_ptr(), h.contiguous().data_ptr(),
+                _f32flag(h.dtype), _hip().ptr(shared), out.data_ptr(), T, d, top, E)
     return out

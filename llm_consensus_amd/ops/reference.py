@@ -430,3 +430,145 @@ def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions
         o = torch.einsum("grqk,gkv->qgrv", torch.softmax(sc, dim=-1), V)
         out[r0:r1] = o.reshape(r1 - r0, H * Dv)
     return out.to(act_dtype)
+
+
+# ------------------------------------------------------------------ hybrid decoders: pre-norm designs, latent
+# attention, mLSTM, routed feed-forwards
+def sinusoid_rows(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """fp32 [T, 2 * len(inv_freq)]: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i)."""
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    return torch.stack([torch.sin(ang), torch.cos(ang)], -1).reshape(positions.numel(), -1)
+
+
+def add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float, act_dtype):
+    """x (fp32, in place) += y; returns x / sqrt(mean(x^2) + eps) * w in ``act_dtype`` (None without w)."""
+    if y is not None:
+        x.add_(y.float())
+    if w is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(act_dtype)
+
+
+def latent_write(proj: torch.Tensor, col0: int, w: torch.Tensor, eps: float, slot_mapping, cache: torch.Tensor) -> None:
+    """cache [blocks, 1, BS, R] at the rows' slots <- rms_norm(proj[:, col0:col0 + R]) * w."""
+    R, BS = cache.shape[3], cache.shape[2]
+    c = proj[:, col0:col0 + R].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    cache[slots[ok] // BS, 0, slots[ok] % BS, :] = c[ok].to(cache.dtype)
+
+
+def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T, H*K], W [H, N, K] -> y [T, H*N] with y[t, h] = W[h] x[t, h]; ``gate`` [T, H]: y[t, h] *= sigmoid(gate[t, h])."""
+    H, N, K = W.shape
+    y = torch.einsum("thk,hnk->thn", x.float().reshape(x.shape[0], H, K), W.float())
+    if gate is not None:
+        y = y * torch.sigmoid(gate.float())[:, :, None]
+    return y.reshape(x.shape[0], H * N).to(out_dtype)
+
+
+def capped(x: torch.Tensor, cap: float) -> torch.Tensor:
+    return cap * torch.tanh(x / cap) if cap > 0 else x
+
+
+def mlstm_scan(proj: torch.Tensor, state: torch.Tensor, cu_q, positions, slots, H: int, D: int, Dv: int, cap: float):
+    """Matrix-memory recurrence with a running maximum. proj fp32 [T, >= 2HD + 2HDv + 2H]: columns
+    q | k | v | (output gate) | input-gate logits | forget-gate logits. Per head, with
+    i = cap tanh(. / cap), f = log sigmoid(cap tanh(. / cap)), m <- max(f + m, i):
+    S <- exp(f + m' - m) S + exp(i - m) k [v, 1]^T (the extra column carries the normaliser n),
+    read out with q / sqrt(D). state [slots, H*D*(Dv+1) + H] fp32 (S with n as its last column,
+    then m). Returns (o fp32 [T, H*(Dv+1)] whose last column per head is n.q, m fp32 [T, H])."""
+    T = proj.shape[0]
+    hd, hv = H * D, H * Dv
+    q = proj[:, :hd].float().view(T, H, D) * (D ** -0.5)
+    k = proj[:, hd:2 * hd].float().view(T, H, D)
+    v = torch.cat([proj[:, 2 * hd:2 * hd + hv].float().view(T, H, Dv), torch.ones(T, H, 1, device=proj.device)], -1)
+    ig = capped(proj[:, 2 * hd + 2 * hv:2 * hd + 2 * hv + H].float(), cap)
+    fg = torch.nn.functional.logsigmoid(capped(proj[:, 2 * hd + 2 * hv + H:2 * hd + 2 * hv + 2 * H].float(), cap))
+    out = torch.zeros(T, H, Dv + 1, dtype=torch.float32, device=proj.device)
+    ms = torch.zeros(T, H, dtype=torch.float32, device=proj.device)
+    n_s = H * D * (Dv + 1)
+    for b in range(len(slots)):
+        r0, r1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(slots[b])
+        if slot < 0 or r1 <= r0:
+            continue
+        S = state[slot, :n_s].view(H, D, Dv + 1).clone()
+        m = state[slot, n_s:].clone()
+        if int(positions[r0]) == 0:
+            S.zero_()
+            m.zero_()
+        for t in range(r0, r1):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            a, bb = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+            S = a[:, None, None] * S + (bb[:, None] * k[t])[:, :, None] * v[t][:, None, :]
+            m = mn
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+            ms[t] = m
+        state[slot, :n_s] = S.reshape(-1)
+        state[slot, n_s:] = m
+    return out.view(T, H * (Dv + 1)), ms
+
+
+def mlstm_out(o: torch.Tensor, m: torch.Tensor, w: torch.Tensor, gate: torch.Tensor, H: int, Dv: int, eps: float,
+              act_dtype) -> torch.Tensor:
+    """o [T, H*(Dv+1)] from ``mlstm_scan``: per head h = o[:Dv] / (max(|o[Dv]|, exp(-m)) + 1e-6),
+    h / sqrt(mean(h^2) + eps) * w (w [H*Dv]), times sigmoid(gate)."""
+    T = o.shape[0]
+    oo = o.float().view(T, H, Dv + 1)
+    den = torch.maximum(oo[:, :, Dv].abs(), torch.exp(-m.float())) + 1e-6
+    h = oo[:, :, :Dv] / den[:, :, None]
+    h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)
+    return (h.reshape(T, H * Dv) * w.float() * torch.sigmoid(gate.float())).to(act_dtype)
+
+
+def glu(y: torch.Tensor, act_dtype, kind: str = "relu") -> torch.Tensor:
+    """y [T, 2n] = (gate | up) -> act(gate) * up."""
+    n = y.shape[1] // 2
+    g, u = y[:, :n].float(), y[:, n:].float()
+    g = torch.relu(g) if kind == "relu" else g * torch.sigmoid(g)
+    return (g * u).to(act_dtype)
+
+
+def route_grouped(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
+    """Router over fp32 logits z [T, n]: s = softmax(z); choice = s + correction; the n outputs form
+    ``groups`` equal runs of neighbours, a run's score is its largest choice, only the ``keep`` best runs
+    stay eligible; the ``top`` largest eligible choices are taken (ties: the lower index) with weights
+    s * scale. Returns (ids int32 [T, top], weights fp32 [T, top])."""
+    T, n = z.shape
+    s = torch.softmax(z.float(), -1)
+    ch = s + correction.float()
+    if groups > 1 and keep < groups:
+        gs = ch.view(T, groups, n // groups).max(-1).values
+        order = torch.argsort(gs, dim=-1, descending=True, stable=True)[:, :keep]
+        allow = torch.zeros(T, groups, dtype=torch.bool, device=z.device).scatter_(1, order, True)
+        ch = ch.masked_fill(~allow.repeat_interleave(n // groups, 1), float("-inf"))
+    ids = torch.argsort(ch, dim=-1, descending=True, stable=True)[:, :top]
+    return ids.to(torch.int32), (s.gather(1, ids) * scale).float()
+
+
+def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: torch.Tensor, W: torch.Tensor,
+                   out_dtype, rows: int, relu2_epi: bool = False) -> torch.Tensor:
+    """Sorted position p in [offsets[e], offsets[e+1]) reads x[row_index[p]] (x[p] without an index) and
+    gives W[e] x; W [E, N, K]. Positions of experts >= E (no tensors) stay zero."""
+    E, N, K = W.shape
+    y = torch.zeros(rows, N, dtype=torch.float32, device=x.device)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            xe = x[row_index[lo:hi].long()] if row_index is not None else x[lo:hi]
+            y[lo:hi] = xe.float() @ W[e].float().t()
+    if relu2_epi:
+        y = torch.relu(y).pow(2)
+    return y.to(out_dtype)
+
+
+def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, h: torch.Tensor, E: int,
+            shared: Optional[torch.Tensor]) -> torch.Tensor:
+    """fp32 [T, d]: sum_k wts[t, k] * (ye[slot_of[t, k]] for ids < E, h[t] itself for the identity experts
+    ids >= E) + shared[t]."""
+    T, top = ids.shape
+    rows = ye[slot_of.long()].float().view(T, top, -1)
+    rows = torch.where((ids >= E)[:, :, None], h.float()[:, None, :], rows)
+    out = (rows * wts.float()[:, :, None]).sum(1)
+    return out + shared.float() if shared is not None else out
