@@ -186,3 +186,144 @@ def test_qkv_prep_and_masked_attention(dt, H, G, D, Dv, rot, chunk, window):
         torch.testing.assert_close(tiled.float().cpu(), want,
                                    **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-4, rtol=2e-4)))
     torch.testing.assert_close(got.float().cpu(), want, **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-4, rtol=2e-4)))
+
+
+# ------------------------------------------------------------------ pre-norm designs, latent attention, mLSTM, routing
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("T,d", [(3, 10), (600, 130)])
+def test_scaled_embedding_with_positions_and_the_pre_norm_residual_step(dt, T, d):
+    g = torch.Generator().manual_seed(T)
+    E = torch.randn(37, d, generator=g).to(dt)
+    ids = torch.randint(0, 37, (T,), generator=g).to(torch.int32)
+    pos = torch.randint(0, 5000, (T,), generator=g).to(torch.int32)
+    f = torch.tensor([10000.0 ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64).float()
+    x, _ = ops.embed_rows(ids.to(DEV), E.to(DEV), None, None, 0.37, pos.to(DEV), f.to(DEV))
+    xr, _ = ops.embed_rows(ids, E, None, None, 0.37, pos, f)
+    torch.testing.assert_close(x.cpu(), xr, atol=3e-4, rtol=1e-5)       # fp32 angles of a few thousand radians
+    y, w = torch.randn(T, d, generator=g), torch.rand(d, generator=g) + 0.5
+    xa = ops.add_rmsnorm(x, y.to(DEV), w.to(DEV), 1e-3, dt)
+    want = ref.add_rmsnorm(xr, y, w, 1e-3, dt)
+    torch.testing.assert_close(x.cpu(), xr, atol=3e-4, rtol=1e-5)
+    torch.testing.assert_close(xa.float().cpu(), want.float(), **(_tol(dt) if dt == torch.bfloat16 else dict(atol=3e-4, rtol=1e-4)))
+    assert ops.add_rmsnorm(x, y.to(DEV), None, 1e-3, dt) is None         # the sum alone
+    ref.add_rmsnorm(xr, y, None, 1e-3, dt)
+    torch.testing.assert_close(x.cpu(), xr, atol=3e-4, rtol=1e-5)
+    only = ops.add_rmsnorm(x, None, w.to(DEV), 1e-3, dt)                 # the norm alone
+    torch.testing.assert_close(only.float().cpu(), ref.add_rmsnorm(xr, None, w, 1e-3, dt).float(),
+                               **(_tol(dt) if dt == torch.bfloat16 else dict(atol=3e-4, rtol=1e-4)))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("R", [9, 64, 200])
+def test_latent_write(dt, R):
+    g = torch.Generator().manual_seed(R)
+    T, BS, col0 = 11, 8, 5
+    proj = torch.randn(T, col0 + R + 3, generator=g)
+    w = torch.rand(R, generator=g) + 0.5
+    slots = torch.tensor([3, 9, -1, 0, 17, 22, 23, 8, -1, 30, 31], dtype=torch.int32)
+    c_ref = torch.zeros(4, 1, BS, R, dtype=dt)
+    ref.latent_write(proj, col0, w, 1e-5, slots, c_ref)
+    c = torch.zeros(4, 1, BS, R, dtype=dt, device=DEV)
+    ops.latent_write(proj.to(DEV), col0, w.to(DEV), 1e-5, slots.to(DEV), c)
+    torch.testing.assert_close(c.float().cpu(), c_ref.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("a_dt,w_dt,o_dt", [(torch.float32, torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                            (torch.float32, torch.float32, torch.float32)])
+@pytest.mark.parametrize("M,H,N,K", [(1, 3, 7, 5), (70, 2, 130, 24), (5, 6, 64, 64)])
+def test_head_linear(a_dt, w_dt, o_dt, M, H, N, K):
+    g = torch.Generator().manual_seed(M + N)
+    wide = torch.randn(M, H * K + H + 4, generator=g).to(a_dt)
+    x = wide[:, 2:2 + H * K]                       # a column slice, as the model passes it
+    W = (torch.randn(H, N, K, generator=g) / K ** 0.5).to(w_dt)
+    gate = torch.randn(M, H + 3, generator=g)
+    wd, gd = wide.to(DEV), gate.to(DEV)
+    for gt, gtd in ((None, None), (gate[:, 1:1 + H], gd[:, 1:1 + H])):
+        got = ops.head_linear(wd[:, 2:2 + H * K], W.to(DEV), o_dt, gtd)
+        want = ref.head_linear(x, W, o_dt, gt)
+        torch.testing.assert_close(got.float().cpu(), want.float(), **_tol(o_dt if a_dt == torch.float32 else torch.bfloat16))
+
+
+def _mlstm_case(lens, starts, slots, H, D, Dv, cap, seed, max_len=1):
+    g = torch.Generator().manual_seed(seed)
+    cu, pos, _ = _seqs(lens, starts)
+    slots = torch.tensor(slots, dtype=torch.int32)
+    T = int(cu[-1])
+    proj = torch.randn(T, 2 * H * D + 2 * H * Dv + 2 * H + 3, generator=g)
+    proj[:, 2 * H * D + 2 * H * Dv:] *= 4                                      # gate logits that the cap bends
+    st = torch.randn(4, H * D * (Dv + 1) + H, generator=g)
+    st_ref = st.clone()
+    o_ref, m_ref = ref.mlstm_scan(proj, st_ref, cu, pos, slots, H, D, Dv, cap)
+    sd, pd = st.to(DEV), proj.to(DEV)
+    o, m = ops.mlstm_scan(pd, sd, cu.to(DEV), pos.to(DEV), slots.to(DEV), H, D, Dv, cap, max_len=max_len)
+    live = torch.cat([torch.arange(int(cu[b]), int(cu[b + 1])) for b in range(len(lens)) if int(slots[b]) >= 0])
+    torch.testing.assert_close(o.cpu()[live], o_ref[live], atol=3e-4, rtol=3e-4)
+    torch.testing.assert_close(m.cpu()[live], m_ref[live], atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(sd.cpu(), st_ref, atol=3e-4, rtol=3e-4)
+    wn = torch.rand(H * Dv, generator=g) + 0.5
+    c0 = 2 * H * D + H * Dv
+    for dt in ACTS:
+        y = ops.mlstm_out(o, m, wn.to(DEV), pd[:, c0:c0 + H * Dv], H, Dv, 1e-5, dt)
+        want = ref.mlstm_out(o_ref, m_ref, wn, proj[:, c0:c0 + H * Dv], H, Dv, 1e-5, dt)
+        torch.testing.assert_close(y.float().cpu()[live], want.float()[live],
+                                   **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-3, rtol=2e-3)))
+
+
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 32, 32, 15.0), (3, 24, 70, 2.0), (1, 100, 8, 0.0), (5, 7, 63, 6.0)])
+def test_mlstm_scan_and_read_out(H, D, Dv, cap):
+    """Sequences that start at position 0 (zero state, maximum 0) and that continue from a kept state,
+    a single decoded token, a skipped sequence; more than 64 rows (the maxima come from wave scans of 64)."""
+    _mlstm_case([6, 1, 2, 150, 3], [0, 5, 3, 0, 9], [1, 3, 0, 2, -1], H, D, Dv, cap, seed=D)
+
+
+def test_mlstm_long_portions_run_in_segments():
+    _mlstm_case([300, 129, 5, 200], [40, 0, 7, 3], [1, 0, 3, -1], 2, 24, 70, 8.0, seed=5, max_len=300)
+
+
+@pytest.mark.parametrize("dt", ACTS)
+def test_glu(dt):
+    y = torch.randn(13, 2 * 37, generator=torch.Generator().manual_seed(1))
+    for kind in ("relu", "silu"):
+        torch.testing.assert_close(ops.glu(y.to(DEV), dt, kind).float().cpu(), ref.glu(y, dt, kind).float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("n,top,groups,keep", [(20, 3, 5, 2), (8, 2, 1, 1), (70, 5, 7, 3), (130, 8, 10, 10), (12, 12, 4, 4), (6, 1, 6, 1)])
+def test_route_grouped(n, top, groups, keep):
+    g = torch.Generator().manual_seed(n)
+    T = 75
+    z = torch.randn(T, n, generator=g) * 2
+    corr = torch.randn(n, generator=g) * 0.1 - 0.5                              # choice scores below zero
+    ids, wts = ops.route_grouped(z.to(DEV), corr.to(DEV), top, groups, keep, 1.7)
+    ids_ref, wts_ref = ref.route_grouped(z, corr, top, groups, keep, 1.7)
+    assert (ids.cpu() == ids_ref).all()
+    torch.testing.assert_close(wts.cpu(), wts_ref, atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("x_dt,w_dt", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("T,top,E,I,d,ff", [(1, 2, 3, 1, 10, 7), (90, 3, 5, 2, 40, 20), (200, 4, 40, 0, 24, 70)])
+def test_sorted_expert_products_and_mix(x_dt, w_dt, T, top, E, I, d, ff):
+    g = torch.Generator().manual_seed(T)
+    n = E + I
+    ids = torch.stack([torch.randperm(n, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    wts = torch.rand(T, top, generator=g)
+    x = torch.randn(T, d, generator=g).to(x_dt)
+    up = (torch.randn(E, ff, d, generator=g) / d ** 0.5).to(w_dt)
+    down = (torch.randn(E, d, ff, generator=g) / ff ** 0.5).to(w_dt)
+    shared = torch.randn(T, d, generator=g)
+    off, src, slot = ops.moe_sort(ids.to(DEV), n)
+    off_ref, src_ref, slot_ref = ref_sort = ops.moe_sort(ids, n)
+    assert (off.cpu() == off_ref).all()
+    flat = ids.reshape(-1)
+    sl = slot.cpu().long()
+    assert sorted(sl.tolist()) == list(range(T * top))                                   # a permutation
+    assert ((sl >= off.cpu()[flat.long()]) & (sl < off.cpu()[flat.long() + 1])).all()       # inside its expert's range
+    assert (src.cpu()[sl] == torch.arange(T * top) // top).all()
+    act = ops.grouped_linear(x.to(DEV), src, off, up.to(DEV), x_dt, T * top, relu2_epi=True)
+    ye = ops.grouped_linear(act, None, off, down.to(DEV), torch.float32, T * top)
+    got = ops.moe_mix(ye, slot, ids.to(DEV), wts.to(DEV), x.to(DEV), E, shared.to(DEV))
+    act_ref = ref.grouped_linear(x, src_ref, off_ref, up, x_dt, T * top, relu2_epi=True)
+    ye_ref = ref.grouped_linear(act_ref, None, off_ref, down, torch.float32, T * top)
+    want = ref.moe_mix(ye_ref, slot_ref, ids, wts, x, E, shared)
+    torch.testing.assert_close(got.cpu(), want, **(dict(atol=5e-2, rtol=5e-2) if x_dt == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
+    none = ops.moe_mix(ye, slot, ids.to(DEV), wts.to(DEV), x.to(DEV), E, None)
+    torch.testing.assert_close(none.cpu(), want - shared, **(dict(atol=5e-2, rtol=5e-2) if x_dt == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
