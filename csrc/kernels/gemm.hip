@@ -301,6 +301,10 @@ LC_EXPORT int lc_gemm_grouped(const void* Wp_all, long long expert_stride, const
     gemm_grouped_kernel<EPI_BF16><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
   else if (epi == EPI_SWIGLU)
     gemm_grouped_kernel<EPI_SWIGLU><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
+  else if (epi == EPI_RELU2)
+    gemm_grouped_kernel<EPI_RELU2><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
+  else if (epi == EPI_F32)
+    gemm_grouped_kernel<EPI_F32><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
   else
     return -2;
   LC_RETURN_LAST_ERROR();

@@ -9,6 +9,7 @@ enum Epilogue : int {
   EPI_BF16 = 0,    // Y bf16 [M, ldy]  (+bias)
   EPI_F32 = 1,     // Y f32  [M, ldy]  (+bias); with split-K: slab blockIdx.y of [S, M, ldy], no bias
   EPI_SWIGLU = 2,  // n-tiles alternate gate/up; Y bf16 [M, N/2] = silu(gate)*up (+bias before act)
+  EPI_RELU2 = 3,   // Y bf16 [M, ldy] = relu(. + bias)^2 (the grouped kernels)
 };
 
 LC_DEVICE float silu(float x) { return x / (1.f + __expf(-x)); }
@@ -44,7 +45,14 @@ LC_DEVICE void store_tile(const f32x4& acc, const f32x4* acc_up, void* __restric
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) v[r] = acc[r] + ((bias && nb + r < N) ? bf16_to_f32(bias[nb + r]) : 0.f);
-    if constexpr (EPI == EPI_BF16) {
+    if constexpr (EPI == EPI_RELU2) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = fmaxf(v[r], 0.f);
+        v[r] *= v[r];
+      }
+    }
+    if constexpr (EPI == EPI_BF16 || EPI == EPI_RELU2) {
       bf16_t* dst = static_cast<bf16_t*>(Y) + static_cast<size_t>(m) * ldy + nb;
       if (nb + 3 < N) {
         u32x2 o;

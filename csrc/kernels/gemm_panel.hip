@@ -547,7 +547,8 @@ __global__ __launch_bounds__(512) void gemm_panel_grouped_kernel(const bf16_t* _
 
   const int nbase = blockIdx.x * GP_BN + wn * (S::NT_W * 16), mbase = wm * (S::MT_W * 16);
   // rows of this expert start at r0 in the output; SwiGLU halves the column count
-  bf16_t* Ye = static_cast<bf16_t*>(Y) + static_cast<size_t>(r0) * ldy;
+  void* Ye = EPI == EPI_F32 ? static_cast<void*>(static_cast<float*>(Y) + static_cast<size_t>(r0) * ldy)
+                            : static_cast<void*>(static_cast<bf16_t*>(Y) + static_cast<size_t>(r0) * ldy);
 #pragma unroll
   for (int i = 0; i < S::NT_W; ++i)
 #pragma unroll
@@ -575,11 +576,19 @@ int launch_panel_grouped(int epi, const bf16_t* w, long long stride, const bf16_
                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_panel_grouped_kernel<BM, EPI_SWIGLU>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_panel_grouped_kernel<BM, EPI_RELU2>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_panel_grouped_kernel<BM, EPI_F32>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   });
   if (epi == EPI_BF16)
     gemm_panel_grouped_kernel<BM, EPI_BF16><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
   else if (epi == EPI_SWIGLU)
     gemm_panel_grouped_kernel<BM, EPI_SWIGLU><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+  else if (epi == EPI_RELU2)
+    gemm_panel_grouped_kernel<BM, EPI_RELU2><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+  else if (epi == EPI_F32)
+    gemm_panel_grouped_kernel<BM, EPI_F32><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
   else
     return -2;
   return static_cast<int>(hipGetLastError());

@@ -31,13 +31,22 @@ __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* _
   const typename Act<EF32>::type* e = static_cast<const typename Act<EF32>::type*>(E) + static_cast<size_t>(id) * d;
   typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
   // optional sinusoidal position vector: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i), fp32 angles
-  const float pos = inv_freq != nullptr ? static_cast<float>(positions[row]) : 0.f;
-  for (int c = lane; c < d; c += 64) {
-    float v = Act<EF32>::load(e, c) * scale;
-    if (inv_freq != nullptr) {
-      const float ang = pos * inv_freq[c >> 1];
-      v += (c & 1) ? cosf(ang) : sinf(ang);
+  if (inv_freq != nullptr) {                      // a lane owns the (sin, cos) pair of one angle; d is even
+    const float pos = static_cast<float>(positions[row]);
+    for (int i = lane; 2 * i < d; i += 64) {
+      float sn, cs;
+      sincosf(pos * inv_freq[i], &sn, &cs);
+      const float v0 = Act<EF32>::load(e, 2 * i) * scale + sn, v1 = Act<EF32>::load(e, 2 * i + 1) * scale + cs;
+      *reinterpret_cast<float2*>(x + static_cast<size_t>(row) * d + 2 * i) = make_float2(v0, v1);
+      if (a != nullptr) {
+        Act<AF32>::store(a, static_cast<size_t>(row) * d + 2 * i, v0);
+        Act<AF32>::store(a, static_cast<size_t>(row) * d + 2 * i + 1, v1);
+      }
     }
+    return;
+  }
+  for (int c = lane; c < d; c += 64) {
+    const float v = Act<EF32>::load(e, c) * scale;
     x[static_cast<size_t>(row) * d + c] = v;
     if (a != nullptr) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, v);
   }
@@ -77,11 +86,13 @@ __global__ __launch_bounds__(256) void scalar_norm_add_kernel(float* __restrict_
   }
 }
 
+// out [T, cols] = relu(y[:, :cols])^2 for y of row stride ld.
 template <bool AF32>
-__global__ void relu2_kernel(const float* __restrict__ y, void* __restrict__ out, long long n) {
+__global__ void relu2_kernel(const float* __restrict__ y, void* __restrict__ out, long long n, int cols, int ld) {
   const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float v = fmaxf(y[i], 0.f);
+  const long long t = i / cols;
+  const float v = fmaxf(y[t * ld + (i - t * cols)], 0.f);
   Act<AF32>::store(static_cast<typename Act<AF32>::type*>(out), i, v * v);
 }
 
@@ -503,7 +514,7 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(
 // off when 0). Per tile of 64 keys: lane j scores key lo + 64 * tile + j in fp32 (q from LDS),
 // online softmax across the wave, then the lanes split the value columns and walk the tile's
 // keys (weights and cache rows from LDS). Serves prompt portions and single decoded tokens.
-constexpr int kMaxVCols = 4;   // value width up to 256
+constexpr int kMaxVCols = 8;   // value width up to 512
 
 template <bool CF32, bool AF32>
 __global__ __launch_bounds__(256) void attn_masked_kernel(
@@ -862,13 +873,28 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict
   const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A) + static_cast<size_t>(h) * K;
   const typename Act<WF32>::type* w = static_cast<const typename Act<WF32>::type*>(W) + static_cast<size_t>(h) * N * K;
   float acc[4][4] = {};
-  for (int k0 = 0; k0 < K; k0 += 16) {
-    for (int i = threadIdx.x; i < 64 * 16; i += 256) {
+  // a thread stages four elements of each operand per slab; the next slab's are loaded into registers
+  // before the current one is multiplied, so the loads' latency hides behind the products
+  float ra[4], rw[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = threadIdx.x + 256 * j;
       const int r = i >> 4, k = i & 15;
-      As[k][r] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * lda + k0 + k) : 0.f;
-      Ws[k][r] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
+      ra[j] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * lda + k0 + k) : 0.f;
+      rw[j] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      As[i & 15][i >> 4] = ra[j];
+      Ws[i & 15][i >> 4] = rw[j];
     }
     __syncthreads();
+    if (k0 + 16 < K) fetch(k0 + 16);
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       float av[4], wv[4];
@@ -938,11 +964,14 @@ LC_EXPORT int lc_scalar_norm_add(void* x, const void* y, const void* gain, float
   LC_RETURN_LAST_ERROR();
 }
 
-LC_EXPORT int lc_relu2(const void* y, void* out, int act_f32, long long n, hipStream_t st) {
-  if (n <= 0) return 0;
+// y [T, >= cols] with row stride ld -> out [T, cols].
+LC_EXPORT int lc_relu2(const void* y, void* out, int act_f32, int T, int cols, int ld, hipStream_t st) {
+  if (T <= 0 || cols <= 0) return 0;
+  if (ld < cols) return -1;
+  const long long n = static_cast<long long>(T) * cols;
   const dim3 grid(static_cast<unsigned>((n + 255) / 256)), block(256);
-  if (act_f32) relu2_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n);
-  else relu2_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n);
+  if (act_f32) relu2_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n, cols, ld);
+  else relu2_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, n, cols, ld);
   LC_RETURN_LAST_ERROR();
 }
 

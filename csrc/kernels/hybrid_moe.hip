@@ -11,12 +11,13 @@ constexpr int kMaxTop = 32;
 constexpr int kMaxGroups = 64;
 
 // ---------------------------------------------------------------- routing
-// One wave per token. z [T, n] fp32 router logits. s = softmax(z); choice = s + correction; the n
+// One wave per token. z [T, n] fp32 router logits (row stride ld). s = softmax(z); choice = s + correction; the n
 // outputs form ``groups`` runs of n / groups neighbours, a run's score is its largest choice, the
 // ``keep`` best runs stay eligible (ties: the lower index); the ``top`` largest eligible choices are
 // taken (ties: the lower index) with weights s * scale.
-__global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restrict__ z, const float* __restrict__ corr,
-                                                            int T, int n, int top, int groups, int keep, float scale,
+__global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restrict__ z, int ld,
+                                                            const float* __restrict__ corr, int T, int n, int top,
+                                                            int groups, int keep, float scale,
                                                             int32_t* __restrict__ ids, float* __restrict__ wts) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restr
   float* ch = sc + n;                               // choice scores (-inf once taken or not eligible)
   float* gs = ch + n;                               // group scores
   float* ok = gs + kMaxGroups;                      // 1: the group is eligible
-  const float* zr = z + static_cast<size_t>(t) * n;
+  const float* zr = z + static_cast<size_t>(t) * ld;
   float mx = -INFINITY;
   for (int e = lane; e < n; e += 64) mx = fmaxf(mx, zr[e]);
   mx = wave_max(mx);
@@ -242,15 +243,16 @@ __global__ __launch_bounds__(256) void moe_mix_kernel(const float* __restrict__ 
 }  // namespace
 
 // ================================================================= launchers
-LC_EXPORT int lc_route_grouped(const void* z, const void* corr, int T, int n, int top, int groups, int keep, float scale,
-                               void* ids, void* wts, hipStream_t st) {
+LC_EXPORT int lc_route_grouped(const void* z, int ld, const void* corr, int T, int n, int top, int groups, int keep,
+                               float scale, void* ids, void* wts, hipStream_t st) {
   if (T <= 0) return 0;
+  if (ld < n) return -1;
   if (n <= 0 || top <= 0 || top > kMaxTop || top > n || groups <= 0 || groups > kMaxGroups || n % groups || keep < 1 ||
       keep > groups || top > keep * (n / groups))
     return -1;
   const size_t lds = 4 * static_cast<size_t>(2 * n + 2 * kMaxGroups) * sizeof(float);
   if (lds > 64 * 1024) return -1;
-  route_grouped_kernel<<<dim3((T + 3) / 4), dim3(256), lds, st>>>(static_cast<const float*>(z),
+  route_grouped_kernel<<<dim3((T + 3) / 4), dim3(256), lds, st>>>(static_cast<const float*>(z), ld,
                                                                  static_cast<const float*>(corr), T, n, top, groups, keep,
                                                                  scale, static_cast<int32_t*>(ids), static_cast<float*>(wts));
   LC_RETURN_LAST_ERROR();

@@ -1,10 +1,14 @@
-"""Prefill and decode throughput of the Nidozen hybrid decoder beside a Llama-shaped transformer of
-equal width, depth and head sizes (``bench.py --hybrid``). Random weights, synthetic tokens.
+"""Prefill and decode throughput of the hybrid decoders (Nidozen, Telurax) beside each other and a
+Llama-shaped transformer of equal width, depth and head sizes (``bench.py --hybrid``,
+``--hybrid-models telurax,nidozen,llama``). Random weights, synthetic tokens.
 
 Per size: one prompt of ``prompt`` tokens goes through each engine as a single step (prefill
 tokens/s), then ``batch`` requests decode ``new`` tokens each from recorded steps (decode tokens/s).
 The hybrid stack repeats (attention, minGRU, attention on the first layer's keys, minGRU, gated
-linear attention); the transformer has full causal attention and a SwiGLU feed-forward. Prints one
+linear attention); the Telurax stack alternates mLSTM layers with a gated dense feed-forward and
+latent-attention layers (compressed rows of width 128) with a routed feed-forward (32 experts of a
+sixteenth of the dense width plus 4 identity experts in 4 groups of which 2 are kept, 4 chosen, a shared
+expert of a quarter); the transformer has full causal attention and a SwiGLU feed-forward. Prints one
 JSON line. Per-kernel times come from running this under ``rocprofv3 --kernel-trace --stats``.
 """
 from __future__ import annotations
@@ -48,6 +52,26 @@ def hybrid_config(s: dict):
                                                      "rank": 64}, "mlp": {"kind": "dense", "ff": s["ff"]}})
     return config_from_dict({"architecture": "Nidozen", "vocab": s["vocab"], "width": s["width"],
                              "norm": {"eps": 1e-5}, "layers": layers}, name="nidozen-bench")
+
+
+def telurax_config(s: dict):
+    from .models.hybrid import config_from_dict
+
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            layers.append({"type": "mlstm", "mixer": {"heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "gate_cap": 15.0},
+                           "mlp": {"kind": "dense", "ff": s["ff"]}})
+        else:
+            layers.append({"type": "latent_attention",
+                           "mixer": {"heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "kv_rank": 128,
+                                     "scale": s["dim"] ** -0.5},
+                           "mlp": {"kind": "moe", "expert": {"ff": s["ff"] // 16},
+                                   "router": {"experts": 32, "identity": 4, "top": 4, "scale": 1.0,
+                                              "groups": {"count": 4, "keep": 2}},
+                                   "shared": {"ff": s["ff"] // 4}}})
+    return config_from_dict({"architecture": "Telurax", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5},
+                             "embedding": {"scale": 1.0}, "logit_scale": 1.0, "layers": layers}, name="telurax-bench")
 
 
 def transformer_config(s: dict):
@@ -107,7 +131,7 @@ def run(a) -> int:
 
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    res = {"metric": "prefill / decode tokens per second, Nidozen hybrid beside a Llama-shaped transformer of equal size",
+    res = {"metric": "prefill / decode tokens per second, hybrid decoders beside a Llama-shaped transformer of equal size",
            "dtype": "bf16", "data": "synthetic tokens, random-init weights", "n_gpus": 1,
            "prompt": a.hybrid_prompt, "batch": a.hybrid_batch, "new_tokens": a.hybrid_new, "sizes": {}}
     for name in [n for n in a.hybrid_sizes.split(",") if n]:
@@ -117,6 +141,8 @@ def run(a) -> int:
         for kind in [k for k in a.hybrid_models.split(",") if k]:
             if kind == "nidozen":
                 model = HybridModel.random_init(hybrid_config(s), dev, seed=1)
+            elif kind == "telurax":
+                model = HybridModel.random_init(telurax_config(s), dev, seed=1)
             else:
                 model = TransformerModel.random_init(transformer_config(s), dev, seed=1)
             row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup, phases)
@@ -127,6 +153,9 @@ def run(a) -> int:
             k = ph + "_tokens_per_s"
             if all(k in row.get(m, {}) for m in ("nidozen", "llama")):
                 row[ph + "_ratio"] = row["nidozen"][k] / row["llama"][k]
+            for other in ("nidozen", "llama"):
+                if all(k in row.get(m, {}) for m in ("telurax", other)):
+                    row[f"{ph}_telurax_over_{other}"] = row["telurax"][k] / row[other][k]
         res["sizes"][name] = row
     print(json.dumps(res))
     if a.out:

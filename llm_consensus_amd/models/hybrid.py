@@ -215,8 +215,8 @@ class HybridConfig:
                 raise ValueError(f"{self.name}: layer {i}: unknown mixer {l.type!r} (known: {', '.join(known)})")
             if l.type in ("latent_attention", "mlstm") and (l.heads <= 0 or l.dim <= 0 or l.vdim <= 0):
                 raise ValueError(f"{self.name}: layer {i}: heads, dim and vdim are needed")
-            if l.type == "latent_attention" and (l.kv_rank <= 0 or l.kv_rank > 256):
-                raise ValueError(f"{self.name}: layer {i}: the attention kernels take a latent width of 1..256")
+            if l.type == "latent_attention" and (l.kv_rank <= 0 or l.kv_rank > 512):
+                raise ValueError(f"{self.name}: layer {i}: the attention kernels take a latent width of 1..512")
             if l.type == "mlstm" and (l.dim > 256 or l.gate_cap < 0):
                 raise ValueError(f"{self.name}: layer {i}: mLSTM takes dim <= 256 and a gate cap >= 0")
             if l.moe is not None:
@@ -522,8 +522,8 @@ class HybridLayer:
     value_up: Optional[torch.Tensor] = None         # latent attention: [H, vdim, kv_rank]
     router: Optional[ops.LinearWeight] = None       # routed feed-forward: [experts + identity, d]
     correction: Optional[torch.Tensor] = None       # fp32 [experts + identity]
-    experts_up: Optional[torch.Tensor] = None       # [E, ff, d]
-    experts_down: Optional[torch.Tensor] = None     # [E, d, ff]
+    experts_up: object = None                       # [E, ff, d] row-major, or ops.ExpertWeights (packed for the MFMA kernels)
+    experts_down: object = None                     # [E, d, ff]
     shared_up: Optional[ops.LinearWeight] = None
     shared_down: Optional[ops.LinearWeight] = None
 
@@ -626,12 +626,22 @@ class HybridModel:
             f = p + "mlp."
             if l.moe is not None:
                 e = l.moe
-                kw["router"] = ops.LinearWeight.from_dense(load(f + "router"), None, dev, dtype=dt, plain=True)
-                kw["correction"] = f32(load(f + "correction"))
-                kw["experts_up"] = torch.stack([load(f + f"e{j}.up") for j in range(e.experts)]).to(dt).contiguous()
-                kw["experts_down"] = torch.stack([load(f + f"e{j}.down") for j in range(e.experts)]).to(dt).contiguous()
+                # bf16 operands with fp32 accumulation give the router's logits in 32-bit either way
+                # (and they ride behind the shared expert's up projection, one product for both, if there is one)
                 if e.shared_ff:
-                    kw.update(shared_up=lin(load(f + "shared.up")), shared_down=lin(load(f + "shared.down")))
+                    kw.update(shared_up=lin(torch.cat([load(f + "shared.up"), load(f + "router")], 0)),
+                              shared_down=lin(load(f + "shared.down")))
+                else:
+                    kw["router"] = lin(load(f + "router"))
+                kw["correction"] = f32(load(f + "correction"))
+                ups = torch.stack([load(f + f"e{j}.up") for j in range(e.experts)])
+                downs = torch.stack([load(f + f"e{j}.down") for j in range(e.experts)])
+                if dt == torch.bfloat16 and c.hidden_size % 64 == 0 and e.ff % 64 == 0:
+                    # depths the MFMA kernels take: MFMA fragment order per expert
+                    kw["experts_up"] = ops.ExpertWeights.from_dense(ups, dev)
+                    kw["experts_down"] = ops.ExpertWeights.from_dense(downs, dev)
+                else:
+                    kw["experts_up"], kw["experts_down"] = ups.to(dt).contiguous(), downs.to(dt).contiguous()
             elif l.ff:
                 if c.design.dense_ff == "glu_relu":
                     kw["gate_up"] = lin(torch.cat([load(f + "gate"), load(f + "up")], 0))
@@ -684,6 +694,7 @@ class HybridModel:
             for w in (L.proj, L.out, L.up, L.down, L.decay_up, L.gate_up, L.router, L.shared_up, L.shared_down):
                 n += w.nbytes() if w is not None else 0
             for t in (L.key_up_t, L.value_up, L.experts_up, L.experts_down):
+                t = t.data if isinstance(t, ops.ExpertWeights) else t
                 n += t.numel() * t.element_size() if t is not None else 0
         return n
 
@@ -780,15 +791,18 @@ class HybridModel:
 
     def _routed_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
         e = L.spec.moe
-        z = ops.linear_any(xa, L.router, out_f32=True)
+        shared = None
+        if L.shared_up is not None:
+            su = ops.linear(xa, L.shared_up, out_f32=True)          # shared expert's hidden units | router logits
+            z = su[:, e.shared_ff:e.shared_ff + e.outputs]
+            shared = ops.linear(ops.relu2(su[:, :e.shared_ff], self.dtype), L.shared_down, out_f32=True)
+        else:
+            z = ops.linear(xa, L.router, out_f32=True)
         ids, wts = ops.route_grouped(z, L.correction, e.top, e.groups, e.keep, e.scale)
         offsets, sorted_src, slot_of = ops.moe_sort(ids, e.outputs)
         rows = ids.numel()
         act = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, self.dtype, rows, relu2_epi=True)
         ye = ops.grouped_linear(act, None, offsets, L.experts_down, torch.float32, rows)
-        shared = None
-        if L.shared_up is not None:
-            shared = ops.linear(self._relu2_up(xa, L.shared_up), L.shared_down, out_f32=True)
         return ops.moe_mix(ye, slot_of, ids, wts, xa, e.experts, shared)
 
     def _latent_attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):

@@ -255,7 +255,8 @@ def linear(x: torch.Tensor, w: LinearWeight, out_f32: bool = False, defer_reduce
         return y
     if M > WS_MAX_M:
         tiles256 = ((M + 255) // 256) * (w.n_pad // 256)
-        splits = _choose_gemm256_splits(tiles256, w.k) if (w.n_pad % 256 == 0 and not w.swiglu) else 1
+        # (the reduction of the split-K slabs works on whole groups of 32 columns)
+        splits = _choose_gemm256_splits(tiles256, w.k) if (w.n_pad % 256 == 0 and not w.swiglu and w.n % 32 == 0) else 1
         if splits > 1 and GEMM256_MIN_TILES >= 0:
             # Too few 256x256 tiles to fill the chip (a few hundred rows, narrow output): split K.
             part = torch.empty(splits, M, w.n, dtype=torch.float32, device=x.device)
@@ -291,7 +292,7 @@ def linear(x: torch.Tensor, w: LinearWeight, out_f32: bool = False, defer_reduce
         h.call("lc_gemm256", w.data.data_ptr(), x.data_ptr(), y.data_ptr(), h.ptr(w.bias), M, w.n, w.k, w.n_pad,
                out_n, epi)
         return y
-    kernel, splits, extra = "lc_gemm_panel", _choose_panel_splits(w.n_pad, w.k), (1 if PANEL_DEEP else 0,)
+    kernel, splits, extra = "lc_gemm_panel", _choose_panel_splits(w.n_pad, w.k) if w.n % 32 == 0 else 1, (1 if PANEL_DEEP else 0,)
     if wide:
         extra = (2,)
     if splits == 1:
@@ -950,11 +951,14 @@ def scalar_norm_add(x: torch.Tensor, y: Optional[torch.Tensor], gain: torch.Tens
 
 
 def relu2(y: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+    """relu(y)^2 of an fp32 matrix (may be a column slice of a wider one) in ``act_dtype``."""
     if not y.is_cuda:
         return ref.relu2(y, act_dtype)
-    y = y.contiguous()
-    out = torch.empty(y.shape, dtype=act_dtype, device=y.device)
-    _hip().call("lc_relu2", y.data_ptr(), out.data_ptr(), _f32flag(act_dtype), y.numel())
+    if y.dim() != 2 or y.stride(1) != 1 or y.dtype != torch.float32:
+        raise ValueError("relu2: an fp32 matrix with unit column stride")
+    T, cols = y.shape
+    out = torch.empty(T, cols, dtype=act_dtype, device=y.device)
+    _hip().call("lc_relu2", y.data_ptr(), out.data_ptr(), _f32flag(act_dtype), T, cols, max(y.stride(0), cols))
     return out
 
 
@@ -1216,11 +1220,12 @@ def route_grouped(z: torch.Tensor, correction: torch.Tensor, top: int, groups: i
         raise ValueError("route_grouped: groups must divide the router's width and the kept groups hold `top` outputs")
     if not z.is_cuda:
         return ref.route_grouped(z, correction, top, groups, keep, scale)
-    z = z.contiguous()
+    if z.stride(1) != 1 or z.dtype != torch.float32:
+        raise ValueError("route_grouped: fp32 logits (a column slice of a wider matrix is taken as it is)")
     ids = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
-    _hip().call("lc_route_grouped", z.data_ptr(), correction.data_ptr(), T, n, top, groups, keep, float(scale),
-                ids.data_ptr(), wts.data_ptr())
+    _hip().call("lc_route_grouped", z.data_ptr(), max(z.stride(0), n), correction.data_ptr(), T, n, top, groups, keep,
+                float(scale), ids.data_ptr(), wts.data_ptr())
     return ids, wts
 
 
@@ -1238,13 +1243,28 @@ def moe_sort(ids: torch.Tensor, n: int):
     return offsets, sorted_src, slot_of
 
 
-def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: torch.Tensor, W: torch.Tensor,
+def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: torch.Tensor, W,
                    out_dtype: torch.dtype, rows: int, relu2_epi: bool = False) -> torch.Tensor:
     """Per-expert products over expert-sorted rows: position p in [offsets[e], offsets[e+1]) gives
-    W[e] x[row_index[p]] (x[p] without an index). W [E, N, K] row-major of any shape and type, fp32
-    accumulation; ``relu2_epi``: square of relu. Positions of experts >= E are left unwritten."""
+    W[e] x[row_index[p]] (x[p] without an index); ``relu2_epi``: square of relu. W is either a
+    row-major tensor [E, N, K] of any shape and type (fp32 accumulation on the vector ALUs) or
+    packed ``ExpertWeights`` (bf16 activations, the grouped MFMA kernels: one panel per expert for a
+    few hundred rows, 128 x 128 tiles beyond). Positions of experts >= E are left unwritten."""
+    if isinstance(W, ExpertWeights) and W.data.dim() == 3:
+        W = W.data                                    # CPU: [E, N, K]
     if not x.is_cuda:
         return ref.grouped_linear(x, row_index, offsets, W, out_dtype, rows, relu2_epi)
+    if isinstance(W, ExpertWeights):
+        if x.dtype != torch.bfloat16 or x.shape[1] != W.k or not x.is_contiguous():
+            raise ValueError("grouped_linear: packed experts take contiguous bf16 activations of their depth")
+        if relu2_epi and out_dtype != torch.bfloat16:
+            raise ValueError("grouped_linear: the relu^2 epilogue of the packed kernels writes bf16")
+        y = torch.empty(rows, W.n, dtype=out_dtype, device=x.device)
+        epi = 3 if relu2_epi else (EPI_F32 if out_dtype == torch.float32 else EPI_BF16)
+        gg = "lc_gemm_panel_grouped" if rows <= MOE_PANEL_MAX_ROWS else "lc_gemm_grouped"
+        _hip().call(gg, W.data.data_ptr(), W.data[0].numel(), x.data_ptr(), _hip().ptr(row_index), offsets.data_ptr(),
+                    W.data.shape[0], y.data_ptr(), int(rows), W.n, W.k, W.n_pad, W.n, epi)
+        return y
     E, N, K = W.shape
     if x.shape[1] != K or x.stride(1) != 1 or not W.is_contiguous():
         raise ValueError("grouped_linear: activations of the experts' depth")

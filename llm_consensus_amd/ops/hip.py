@@ -60,7 +60,7 @@ _SIGNATURES = {
     # hybrid decoders (hybrid.hip)
     "lc_embed_rows": [_P, _P, _I, _P, _P, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P],
     "lc_scalar_norm_add": [_P, _P, _P, _F, _P, _I, _I, _I, _P],
-    "lc_relu2": [_P, _P, _I, _L, _P],
+    "lc_relu2": [_P, _P, _I, _I, _I, _I, _P],
     "lc_mingru_scan": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
     "lc_gla_scan": [_P, _I, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P],
@@ -74,7 +74,7 @@ _SIGNATURES = {
     "lc_mlstm_scan": [_P, _I, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_glu": [_P, _P, _I, _I, _I, _I, _P],
     # routed feed-forwards of hybrid decoders (hybrid_moe.hip)
-    "lc_route_grouped": [_P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+    "lc_route_grouped": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
     "lc_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P],
     "lc_gemm_any_grouped": [_P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "lc_moe_mix": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _P],

@@ -327,3 +327,23 @@ def test_sorted_expert_products_and_mix(x_dt, w_dt, T, top, E, I, d, ff):
     torch.testing.assert_close(got.cpu(), want, **(dict(atol=5e-2, rtol=5e-2) if x_dt == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
     none = ops.moe_mix(ye, slot, ids.to(DEV), wts.to(DEV), x.to(DEV), E, None)
     torch.testing.assert_close(none.cpu(), want - shared, **(dict(atol=5e-2, rtol=5e-2) if x_dt == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
+
+
+@pytest.mark.parametrize("T,top,E,d,ff", [(5, 2, 3, 64, 64), (100, 3, 6, 128, 192), (400, 4, 9, 64, 128)])
+def test_sorted_expert_products_on_the_packed_mfma_kernels(T, top, E, d, ff):
+    """bf16 experts whose depths are multiples of 64 go through the grouped MFMA kernels (a panel per expert up to a few
+    hundred routed rows, tiles beyond) with the relu^2 and fp32 epilogues; experts past E get no rows written."""
+    g = torch.Generator().manual_seed(T)
+    n = E + 2
+    ids = torch.stack([torch.randperm(n, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    up = (torch.randn(E, ff, d, generator=g) / d ** 0.5).to(torch.bfloat16)
+    down = (torch.randn(E, d, ff, generator=g) / ff ** 0.5).to(torch.bfloat16)
+    off, src, slot = ops.moe_sort(ids.to(DEV), n)
+    act = ops.grouped_linear(x.to(DEV), src, off, ops.ExpertWeights.from_dense(up, DEV), torch.bfloat16, T * top, relu2_epi=True)
+    ye = ops.grouped_linear(act, None, off, ops.ExpertWeights.from_dense(down, DEV), torch.float32, T * top)
+    act_ref = ref.grouped_linear(x, src.cpu(), off.cpu(), up, torch.bfloat16, T * top, relu2_epi=True)
+    ye_ref = ref.grouped_linear(act_ref, None, off.cpu(), down, torch.float32, T * top)
+    real = int(off.cpu()[E])
+    torch.testing.assert_close(act.float().cpu()[:real], act_ref.float()[:real], atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(ye.cpu()[:real], ye_ref[:real], atol=3e-2, rtol=3e-2)

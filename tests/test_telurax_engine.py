@@ -113,6 +113,7 @@ def test_the_registry_names_the_designs_of_the_model_code():
     ("latent attention", [latent(), latent(heads=1, dim=7, vdim=5, rank=9, scale=1.1)]),
     ("latent widths the matrix-core kernel takes", [latent(heads=4, dim=16, vdim=16, rank=32), latent(heads=2, dim=8, vdim=24, rank=16)]),
     ("latent wider than a wave", [latent(heads=2, dim=8, vdim=8, rank=72)]),
+    ("latent wider than the width", [latent(heads=2, dim=8, vdim=8, rank=300)]),
     ("mlstm", [mlstm(), mlstm(heads=3, dim=5, vdim=33, cap=2.0)]),
     ("mlstm without a cap, one head", [mlstm(heads=1, dim=40, vdim=3, cap=0.0)]),
     ("gated dense feed-forward", [mlstm(mlp=dense()), latent(mlp=dense(9))]),
@@ -132,6 +133,20 @@ def test_depths_the_mfma_products_take(device, dtype):
     cfg = config([latent(heads=2, dim=32, vdim=32, rank=64, mlp=dense(128)), mlstm(heads=2, dim=32, vdim=32, mlp=moe(ff=64, shared=64)),
                   latent(heads=4, dim=16, vdim=16, rank=32, mlp=moe(shared=0))], width=64, vocab=70)
     _whole_prompt(cfg, device, dtype, "mfma depths", cuts=[40, 2, 17])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_deep_products_whose_outputs_are_no_multiple_of_32(device, dtype):
+    """Width 1024: deep enough that the bf16 MFMA products of a few rows (and of a few hundred) split
+    their depth over workgroups, while the fused projections, the vocabulary and the router have
+    widths like 90 or 179. A long portion, a short one and decoded tokens."""
+    cfg = config([latent(heads=3, dim=16, vdim=16, rank=32, mlp=moe(ff=64, shared=64)), mlstm(heads=2, dim=16, vdim=24, mlp=dense(64))],
+                 width=1024, vocab=90)
+    eng, W = build(cfg, device, dtype, blocks=24)
+    toks = tokens(300, cfg["vocab"], 3)
+    got = replay_alone(eng, toks, [270, 20])
+    assert rel_err(got, oracle.forward(cfg, W, toks), calls(dtype, len(toks))) < limit(dtype)
 
 
 @pytest.mark.parametrize("device", DEVICES)
