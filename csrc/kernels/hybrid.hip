@@ -861,50 +861,63 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ 
 // C[m, h, :] = W[h] A[m, h, :] for H heads side by side: A [M, H*K] (row stride lda), W [H, N, K],
 // C [M, H*N]. The tiling of gemm_any_kernel with the head as the third grid dimension. With
 // ``gate`` [M, H] (row stride ld_gate) the head's outputs are scaled by sigmoid(gate[m, h]).
-template <bool AF32, bool WF32, bool CF32>
+// RPT rows per thread: a block covers 16 * RPT rows x 64 columns. Few rows (decode steps) take RPT = 1, which
+// spreads the same products over four times as many waves.
+template <bool AF32, bool WF32, bool CF32, int RPT>
 __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict__ A, int lda, const void* __restrict__ W,
                                                           void* __restrict__ C, const float* __restrict__ gate,
                                                           int ld_gate, int M, int H, int N, int K) {
-  __shared__ float As[16][64 + 4];
-  __shared__ float Ws[16][64 + 4];
+  constexpr int KS = 32;                            // slab depth: per-head depths are short, so few, deep slabs
+  constexpr int TM = 16 * RPT;
+  constexpr int NA = TM * KS / 256, NW = 64 * KS / 256;
+  __shared__ float As[KS][TM + 4];
+  __shared__ float Ws[KS][64 + 4];
   const int h = blockIdx.z;
-  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A) + static_cast<size_t>(h) * K;
   const typename Act<WF32>::type* w = static_cast<const typename Act<WF32>::type*>(W) + static_cast<size_t>(h) * N * K;
-  float acc[4][4] = {};
-  // a thread stages four elements of each operand per slab; the next slab's are loaded into registers
-  // before the current one is multiplied, so the loads' latency hides behind the products
-  float ra[4], rw[4];
+  float acc[RPT][4] = {};
+  // the next slab's elements are loaded into registers before the current one is multiplied, so the
+  // loads' latency hides behind the products
+  float ra[NA], rw[NW];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NA; ++j) {
       const int i = threadIdx.x + 256 * j;
-      const int r = i >> 4, k = i & 15;
+      const int r = i / KS, k = i % KS;
       ra[j] = (m0 + r < M && k0 + k < K) ? Act<AF32>::load(a, static_cast<size_t>(m0 + r) * lda + k0 + k) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      const int r = i / KS, k = i % KS;
       rw[j] = (n0 + r < N && k0 + k < K) ? Act<WF32>::load(w, static_cast<size_t>(n0 + r) * K + k0 + k) : 0.f;
     }
   };
   fetch(0);
-  for (int k0 = 0; k0 < K; k0 += 16) {
+  for (int k0 = 0; k0 < K; k0 += KS) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NA; ++j) {
       const int i = threadIdx.x + 256 * j;
-      As[i & 15][i >> 4] = ra[j];
-      Ws[i & 15][i >> 4] = rw[j];
+      As[i % KS][i / KS] = ra[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      Ws[i % KS][i / KS] = rw[j];
     }
     __syncthreads();
-    if (k0 + 16 < K) fetch(k0 + 16);
+    if (k0 + KS < K) fetch(k0 + KS);
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      float av[4], wv[4];
+    for (int k = 0; k < KS; ++k) {
+      float av[RPT], wv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        av[i] = As[k][ty * 4 + i];
-        wv[i] = Ws[k][tx * 4 + i];
-      }
+      for (int i = 0; i < RPT; ++i) av[i] = As[k][ty * RPT + i];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i) wv[i] = Ws[k][tx * 4 + i];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * wv[j];
     }
@@ -912,8 +925,8 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict
   }
   typename Act<CF32>::type* c = static_cast<typename Act<CF32>::type*>(C);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = m0 + ty * 4 + i;
+  for (int i = 0; i < RPT; ++i) {
+    const int r = m0 + ty * RPT + i;
     if (r >= M) continue;
     const float g = gate != nullptr ? sigmoidf_(gate[static_cast<size_t>(r) * ld_gate + h]) : 1.f;
 #pragma unroll
@@ -1133,10 +1146,15 @@ LC_EXPORT int lc_head_linear(const void* A, int a_f32, int lda, const void* W, i
                              const void* gate, int ld_gate, int M, int H, int N, int K, hipStream_t st) {
   if (M <= 0 || N <= 0 || H <= 0) return 0;
   if (K <= 0 || lda < H * K || H > 65535 || (gate != nullptr && ld_gate < H)) return -1;
-  const dim3 grid((N + 63) / 64, (M + 63) / 64, H), block(256);
-#define LC_HL(A32, W32, C32)                                                                                   \
-  head_linear_kernel<A32, W32, C32><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, M, H, \
-                                                            N, K)
+  const bool few = M <= 64;                          // decode steps: one row per thread, four times the blocks
+  const dim3 grid((N + 63) / 64, few ? (M + 15) / 16 : (M + 63) / 64, H), block(256);
+#define LC_HL(A32, W32, C32)                                                                                       \
+  if (few)                                                                                                         \
+    head_linear_kernel<A32, W32, C32, 1><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, \
+                                                                 M, H, N, K);                                      \
+  else                                                                                                             \
+    head_linear_kernel<A32, W32, C32, 4><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, \
+                                                                 M, H, N, K)
   const int sel = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
   switch (sel) {
     case 0: LC_HL(false, false, false); break;

@@ -570,7 +570,13 @@ class HybridModel:
                                  f"{tuple(shapes[name])}")
             return t.to(dev)
 
-        def lin(W: torch.Tensor, b: Optional[torch.Tensor] = None) -> ops.LinearWeight:
+        def lin(W: torch.Tensor, b: Optional[torch.Tensor] = None, pad: bool = False) -> ops.LinearWeight:
+            # ``pad``: zero rows up to a multiple of 32 outputs, for fused projections whose consumers
+            # address their columns anyway (products that split their depth reduce whole groups of 32 columns)
+            extra = -W.shape[0] % 32 if pad else 0
+            if extra:
+                W = torch.cat([W, W.new_zeros(extra, W.shape[1])], 0)
+                b = torch.cat([b, b.new_zeros(extra)], 0) if b is not None else None
             return ops.LinearWeight.from_dense(W, b, dev, dtype=dt, any_shape=True)
 
         def f32(t: torch.Tensor) -> torch.Tensor:
@@ -612,7 +618,7 @@ class HybridModel:
                 out = lin(load(m + "o"))
             elif l.type == "latent_attention":
                 # queries | compressed row | one gate logit per head, in one product
-                proj = lin(torch.cat([load(m + n) for n in ("q", "dkv", "g")], 0))
+                proj = lin(torch.cat([load(m + n) for n in ("q", "dkv", "g")], 0), pad=True)
                 kw["latent_norm"] = f32(load(m + "dkv.norm"))
                 kw["key_up_t"] = load(m + "uk").view(l.heads, l.dim, l.kv_rank).transpose(1, 2).to(dt).contiguous()
                 kw["value_up"] = load(m + "uv").view(l.heads, l.vdim, l.kv_rank).to(dt).contiguous()
@@ -620,7 +626,7 @@ class HybridModel:
             else:
                 hd, hv = l.heads * l.dim, l.heads * l.vdim
                 bias = torch.cat([torch.zeros(2 * hd + 2 * hv, device=dev), load(m + "i.b"), load(m + "f.b")])
-                proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "i", "f")], 0), bias)
+                proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v", "g", "i", "f")], 0), bias, pad=True)
                 kw["head_norm"] = f32(load(m + "norm"))
                 out = lin(load(m + "o"))
             f = p + "mlp."
@@ -629,7 +635,7 @@ class HybridModel:
                 # bf16 operands with fp32 accumulation give the router's logits in 32-bit either way
                 # (and they ride behind the shared expert's up projection, one product for both, if there is one)
                 if e.shared_ff:
-                    kw.update(shared_up=lin(torch.cat([load(f + "shared.up"), load(f + "router")], 0)),
+                    kw.update(shared_up=lin(torch.cat([load(f + "shared.up"), load(f + "router")], 0), pad=True),
                               shared_down=lin(load(f + "shared.down")))
                 else:
                     kw["router"] = lin(load(f + "router"))
