@@ -18,7 +18,7 @@ template <bool EF32, bool AF32>
 __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* __restrict__ E, float* __restrict__ x,
                                   void* __restrict__ xa, int T, int d, int vocab, const int32_t* __restrict__ feed_tok,
                                   const int32_t* __restrict__ feed_rows, float scale,
-                                  const int32_t* __restrict__ positions, const float* __restrict__ inv_freq) {
+                                  const int32_t* __restrict__ positions, const double* __restrict__ inv_freq) {
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= T) return;
@@ -30,12 +30,16 @@ __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const void* _
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const typename Act<EF32>::type* e = static_cast<const typename Act<EF32>::type*>(E) + static_cast<size_t>(id) * d;
   typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
-  // optional sinusoidal position vector: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i), fp32 angles
+  // optional sinusoidal position vector: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i), f an fp64 table
   if (inv_freq != nullptr) {                      // a lane owns the (sin, cos) pair of one angle; d is even
-    const float pos = static_cast<float>(positions[row]);
+    // the angle p * f and its reduction to [-pi, pi] in fp64 (thousands of radians would cost an fp32
+    // angle four digits), sine and cosine of the reduced angle in fp32
+    const double pos = static_cast<double>(positions[row]);
     for (int i = lane; 2 * i < d; i += 64) {
+      const double ang = pos * inv_freq[i];
+      const double red = ang - 6.283185307179586476925 * rint(ang * 0.159154943091895335769);
       float sn, cs;
-      sincosf(pos * inv_freq[i], &sn, &cs);
+      sincosf(static_cast<float>(red), &sn, &cs);
       const float v0 = Act<EF32>::load(e, 2 * i) * scale + sn, v1 = Act<EF32>::load(e, 2 * i + 1) * scale + cs;
       *reinterpret_cast<float2*>(x + static_cast<size_t>(row) * d + 2 * i) = make_float2(v0, v1);
       if (a != nullptr) {
@@ -951,7 +955,7 @@ LC_EXPORT int lc_embed_rows(const void* ids, const void* E, int e_f32, void* x, 
                                                       xa, T, d, vocab, static_cast<const int32_t*>(feed_tok), \
                                                       static_cast<const int32_t*>(feed_rows), scale,          \
                                                       static_cast<const int32_t*>(positions),                 \
-                                                      static_cast<const float*>(inv_freq))
+                                                      static_cast<const double*>(inv_freq))
   if (e_f32 && act_f32) LC_EMB(true, true);
   else if (e_f32) LC_EMB(true, false);
   else if (act_f32) LC_EMB(false, true);

@@ -549,11 +549,11 @@ class HybridModel:
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self._max_len = 1
         self._portions = (0, 0)
-        self.pos_freq: Optional[torch.Tensor] = None    # fp32 [d/2]: frequencies of the sinusoidal position vector
+        self.pos_freq: Optional[torch.Tensor] = None    # fp64 [d/2]: frequencies of the sinusoidal position vector
         if cfg.design.pos_base > 0:
             half = cfg.hidden_size // 2
             f = torch.tensor([cfg.design.pos_base ** (-2.0 * j / cfg.hidden_size) for j in range(half)], dtype=torch.float64)
-            self.pos_freq = f.to(torch.float32).to(self.device)
+            self.pos_freq = f.to(self.device)
 
     # ------------------------------------------------------------------ construction
     def set_weights(self, get) -> None:

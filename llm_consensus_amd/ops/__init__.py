@@ -907,11 +907,11 @@ def embed_rows(ids: torch.Tensor, E: torch.Tensor, act_dtype: Optional[torch.dty
                positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None):
     """Rows E[ids] * scale as (fp32 [T, d], copy in ``act_dtype`` or None). E is bf16 or fp32; with
     ``act_dtype`` fp32 the copy IS the fp32 tensor. ``feed`` as in ``embed``. With ``positions`` and
-    ``inv_freq`` (fp32 [d/2]) a sinusoidal position vector is added: entry 2i is sin(p f_i), entry
-    2i + 1 cos(p f_i), angles in fp32. Also the row gather of an fp32 matrix."""
+    ``inv_freq`` (fp64 [d/2]) a sinusoidal position vector is added: entry 2i is sin(p f_i), entry
+    2i + 1 cos(p f_i), the angle and its reduction in fp64. Also the row gather of an fp32 matrix."""
     T, d = ids.numel(), E.shape[1]
-    if inv_freq is not None and (positions is None or 2 * inv_freq.numel() != d):
-        raise ValueError("embed_rows: the position table needs positions and d / 2 frequencies")
+    if inv_freq is not None and (positions is None or 2 * inv_freq.numel() != d or inv_freq.dtype != torch.float64):
+        raise ValueError("embed_rows: the position table needs positions and d / 2 fp64 frequencies")
     if not ids.is_cuda:
         if feed is not None:
             tok, rows = feed

@@ -435,9 +435,9 @@ def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions
 # ------------------------------------------------------------------ hybrid decoders: pre-norm designs, latent
 # attention, mLSTM, routed feed-forwards
 def sinusoid_rows(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
-    """fp32 [T, 2 * len(inv_freq)]: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i)."""
-    ang = positions.float()[:, None] * inv_freq.float()[None, :]
-    return torch.stack([torch.sin(ang), torch.cos(ang)], -1).reshape(positions.numel(), -1)
+    """fp32 [T, 2 * len(inv_freq)]: entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i); angles in fp64."""
+    ang = positions.double()[:, None] * inv_freq.double()[None, :]
+    return torch.stack([torch.sin(ang), torch.cos(ang)], -1).reshape(positions.numel(), -1).float()
 
 
 def add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float, act_dtype):
