@@ -455,3 +455,23 @@ model = "h"
     q.write_text("Which? A. a B. b C. c D. d\n")
     assert cli.main(["--config", str(toml), "--questions", str(q), "--device", "cpu", "--no-warm-up"]) == 0
     assert capsys.readouterr().out.strip()[-1] in "ABCD"
+
+
+def test_random_checkpoint_writer_and_random_init(tmp_path):
+    """The family's checkpoint writer and ``random_init`` (benchmarks, stand-ins) know the design's tensors: what
+    one writes the loader reads back, and both models answer the same."""
+    from llm_consensus_amd.models.loader import load_model, write_random_hybrid_checkpoint
+
+    cfg = config_from_dict(config([mlstm(mlp=moe(shared=0)), latent(mlp=dense()), mlstm(), latent(mlp=moe())], width=24, vocab=80))
+    ck = write_random_hybrid_checkpoint(cfg, str(tmp_path / "ck"), seed=7)
+    assert json.loads((ck / "config.json").read_text())["architecture"] == "Telurax"
+    a = load_model(str(ck), "cpu", dtype=torch.float32)
+    b = HybridModel.random_init(cfg, "cpu", seed=7, dtype=torch.float32)
+    assert a.cfg.layers == b.cfg.layers and (a.cfg.embed_scale, a.cfg.logit_scale) == (b.cfg.embed_scale, b.cfg.logit_scale)
+    out = []
+    for m in (a, b):
+        eng = Engine(m, num_kv_blocks=8, block_size=BS, max_batch_seqs=2, state_slots=2, max_model_len=8 * BS,
+                     enable_prefix_cache=False, use_graphs=False, pipeline_decode=False)
+        out.append(replay_alone(eng, tokens(12, 80, 1), [7]))
+    assert np.isfinite(out[0]).all() and np.abs(out[0]).max() > 0
+    np.testing.assert_allclose(out[0], out[1], rtol=1e-6, atol=1e-6)
