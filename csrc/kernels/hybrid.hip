@@ -155,9 +155,11 @@ __global__ void mingru_scan_kernel(const float* __restrict__ zxg, float* __restr
 // state S [D, Dv] in registers (DMAX >= D). q, k and the decay come prepared (gla_prepare_kernel);
 // per token S = a * S + k v^T, o = S^T q.
 // Long portions run as segments of seg_len rows side by side, in three passes:
-//   mode 1  each segment scans its rows from zero; its local state goes to ``cs`` [B, nseg, H, D, Dv]
-//           and the product of its decays to ``ca`` [B, nseg, H, D];
-//   (gla_carry_kernel turns the local states into each segment's incoming state, in place)
+//   scan_segment_state_kernel: what each segment's rows alone add to the state (from zero) goes to
+//           ``cs`` [B, nseg, H, D, Dv] and the product of its decays to ``ca`` [B, nseg, H, D]. No
+//           outputs are needed here, so every state ELEMENT is its own short recurrence and a
+//           thread owns a few of them: thousands of independent chains instead of one per column;
+//   gla_carry_kernel turns the local states into each segment's incoming state, in place;
 //   mode 2  each segment starts from its incoming state, writes its outputs; the last one stores
 //           the sequence's state.
 // mode 0: the whole sequence in one block (decoded tokens, short portions).
@@ -182,8 +184,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, float* __restrict__ out, int H,
                                                       int D, int Dv, int mode, int nseg, int seg_len,
-                                                      float* __restrict__ cs, float* __restrict__ ca,
-                                                      long long state_stride, int ones) {
+                                                      const float* __restrict__ cs, long long state_stride, int ones) {
   const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
   const int dv = blockIdx.x * 64 + threadIdx.x;
   const int slot = slots[b];
@@ -196,14 +197,11 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   float S[DMAX];
   float* st = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * D * Dv;
   const int Dvr = Dv - ones;                      // value columns that come from the projection
-  float* seg_s = cs != nullptr ? cs + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D * Dv : nullptr;
+  const float* seg_s = cs != nullptr ? cs + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D * Dv : nullptr;
   const float* from = mode == 2 ? seg_s : st;
-  const bool zero = mode == 1 || (mode == 0 && positions[q0] == 0);
+  const bool zero = mode == 0 && positions[q0] == 0;
 #pragma unroll
   for (int d = 0; d < DMAX; ++d) S[d] = (!zero && live && d < D) ? from[static_cast<size_t>(d) * Dv + dv] : 0.f;
-  float aprod[(DMAX + 63) / 64];
-#pragma unroll
-  for (int i = 0; i < (DMAX + 63) / 64; ++i) aprod[i] = 1.f;
   // Lane j of the wave loads the prepared operands of key channels j, j + 64, ... of the token (one
   // coalesced 16-byte load per lane, the next token's in flight during the current one); the
   // channel loop then broadcasts them lane by lane (v_readlane) to meet every lane's state column.
@@ -229,7 +227,6 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
     float o = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      aprod[i] *= cur[i].z;                       // this lane's channel of the segment's decay product
 #pragma unroll
       for (int j = 0; j < 64; ++j) {
         const int d = 64 * i + j;
@@ -242,24 +239,78 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
         }
       }
     }
-    if (live && mode != 1) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
+    if (live) out[static_cast<size_t>(t) * H * Dv + h * Dv + dv] = o;
   }
-  if (mode == 1) {
-    if (live) {
-#pragma unroll
-      for (int d = 0; d < DMAX; ++d)
-        if (d < D) seg_s[static_cast<size_t>(d) * Dv + dv] = S[d];
-    }
-    if (blockIdx.x == 0) {
-      float* a = ca + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D;
-#pragma unroll
-      for (int i = 0; i < (DMAX + 63) / 64; ++i)
-        if (threadIdx.x + 64 * i < D) a[threadIdx.x + 64 * i] = aprod[i];
-    }
-  } else if (live && r1 == q1) {
+  if (live && r1 == q1) {
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
       if (d < D) st[static_cast<size_t>(d) * Dv + dv] = S[d];
+  }
+}
+
+// A segment's own contribution to the state, from zero: cs[d, dv] = sum_t (prod_{r > t} a_r[d]) k_t[d] v_t[dv] over
+// its rows, and ca[d] = prod_t a_t[d]. One block per (tile of 32 key channels x 128 value columns, head,
+// sequence x segment); the segment's operands are staged in LDS once (seg_len <= 64 rows), a thread
+// owns 4 x 4 state elements and walks the rows: acc <- a acc + k v.
+constexpr int kSegRows = 64, kSegD = 32, kSegV = 128;
+
+__global__ __launch_bounds__(256) void scan_segment_state_kernel(
+    const float* __restrict__ proj, int ld, const float4* __restrict__ prep, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ slots, int H, int D, int Dv, int nseg, int seg_len, float* __restrict__ cs,
+    float* __restrict__ ca, int ones) {
+  __shared__ float2 ka[kSegRows][kSegD];            // (k, a) of the tile's key channels
+  __shared__ float vs[kSegRows][kSegV];
+  const int b = blockIdx.z / nseg, seg = blockIdx.z % nseg, h = blockIdx.y;
+  const int ndt = (D + kSegD - 1) / kSegD;
+  const int d0 = (blockIdx.x % ndt) * kSegD, v0 = (blockIdx.x / ndt) * kSegV;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (slots[b] < 0 || q1 <= q0) return;
+  const int r0 = q0 + seg * seg_len;
+  if (r0 >= q1) return;                               // the same for the whole block
+  const int n = min(seg_len, q1 - r0);
+  const int Dvr = Dv - ones;
+  for (int i = threadIdx.x; i < kSegRows * kSegD; i += 256) {
+    const int t = i / kSegD, d = d0 + i % kSegD;
+    float2 e = make_float2(0.f, 1.f);                 // rows and channels past the end change nothing
+    if (t < n && d < D) {
+      const float4 x = prep[(static_cast<size_t>(r0 + t) * H + h) * D + d];
+      e = make_float2(x.y, x.z);
+    }
+    ka[t][i % kSegD] = e;
+  }
+  for (int i = threadIdx.x; i < kSegRows * kSegV; i += 256) {
+    const int t = i / kSegV, dv = v0 + i % kSegV;
+    float v = 0.f;
+    if (t < n && dv < Dv) v = dv < Dvr ? proj[static_cast<size_t>(r0 + t) * ld + 2 * H * D + h * Dvr + dv] : 1.f;
+    vs[t][i % kSegV] = v;
+  }
+  __syncthreads();
+  const int td = (threadIdx.x >> 5) * 4, tv = threadIdx.x & 31;   // channels td .. td + 3, columns tv + 32 j
+  float acc[4][4] = {};
+  float ap[4] = {1.f, 1.f, 1.f, 1.f};
+  for (int t = 0; t < n; ++t) {
+    float vv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) vv[j] = vs[t][tv + 32 * j];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 e = ka[t][td + i];
+      ap[i] *= e.y;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = e.y * acc[i][j] + e.x * vv[j];
+    }
+  }
+  float* out = cs + ((static_cast<size_t>(b) * nseg + seg) * H + h) * D * Dv;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = d0 + td + i;
+    if (d >= D) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int dv = v0 + tv + 32 * j;
+      if (dv < Dv) out[static_cast<size_t>(d) * Dv + dv] = acc[i][j];
+    }
+    if (v0 == 0 && tv == 0) ca[((static_cast<size_t>(b) * nseg + seg) * H + h) * D + d] = ap[i];
   }
 }
 
@@ -1045,14 +1096,18 @@ static int launch_linear_scan(const void* proj, int ld, const void* prep, void* 
                                                 static_cast<float*>(state), static_cast<const int32_t*>(cu_q),      \
                                                 static_cast<const int32_t*>(positions),                             \
                                                 static_cast<const int32_t*>(slots), static_cast<float*>(out), H, D, \
-                                                Dv, MODE, nseg, kScanSegment, cs, ca, state_stride, ones)
+                                                Dv, MODE, nseg, kScanSegment, cs, state_stride, ones)
 #define LC_GLA_D(MODE)          \
   if (D <= 32) LC_GLA(32, MODE);  \
   else if (D <= 64) LC_GLA(64, MODE); \
   else if (D <= 128) LC_GLA(128, MODE); \
   else LC_GLA(256, MODE)
   if (segmented) {
-    LC_GLA_D(1);
+    static_assert(kScanSegment <= kSegRows, "a segment's rows are staged in LDS at once");
+    const dim3 sgrid(((D + kSegD - 1) / kSegD) * ((Dv + kSegV - 1) / kSegV), H, B * nseg);
+    scan_segment_state_kernel<<<sgrid, dim3(256), 0, st>>>(
+        static_cast<const float*>(proj), ld, static_cast<const float4*>(prep), static_cast<const int32_t*>(cu_q),
+        static_cast<const int32_t*>(slots), H, D, Dv, nseg, kScanSegment, cs, ca, ones);
     const size_t n = static_cast<size_t>(H) * D * Dv;
     gla_carry_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256), B), dim3(256), 0, st>>>(
         cs, ca, static_cast<const float*>(state), static_cast<const int32_t*>(cu_q),
