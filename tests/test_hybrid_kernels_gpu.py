@@ -269,7 +269,7 @@ def _mlstm_case(lens, starts, slots, H, D, Dv, cap, seed, max_len=1):
                                    **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-3, rtol=2e-3)))
 
 
-@pytest.mark.parametrize("H,D,Dv,cap", [(2, 32, 32, 15.0), (3, 24, 70, 2.0), (1, 100, 8, 0.0), (5, 7, 63, 6.0)])
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 32, 32, 15.0), (3, 24, 70, 2.0), (1, 100, 8, 0.0), (5, 7, 63, 6.0), (2, 160, 40, 5.0)])
 def test_mlstm_scan_and_read_out(H, D, Dv, cap):
     """Sequences that start at position 0 (zero state, maximum 0) and that continue from a kept state,
     a single decoded token, a skipped sequence; more than 64 rows (the maxima come from wave scans of 64)."""
