@@ -963,7 +963,7 @@ def relu2(y: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
 
 
 def _scan_scratch(B: int, max_len: int, state_floats: int, decay_floats: int, device) -> Optional[torch.Tensor]:
-    """Carry buffer of the segmented scans (portions longer than two segments of 64 rows run as
+    """Carry buffer of the segmented scans (portions longer than two segments of 32 rows run as
     segments side by side: hybrid.hip), None when the step's portions are short."""
     n = int(_hip().lib().lc_scan_scratch_floats(B, int(max_len), state_floats, decay_floats))
     return torch.empty(n, dtype=torch.float32, device=device) if n else None

@@ -88,7 +88,7 @@ def test_mingru_scan(dt, w):
 
 @pytest.mark.parametrize("dt", ACTS)
 def test_scans_of_long_portions_run_in_segments(dt):
-    """Portions longer than two segments of 64 rows take the three-pass form: same results, with a
+    """Portions longer than two segments of 32 rows take the three-pass form: same results, with a
     portion that starts from a kept state, one that starts at position 0, a short one and a skipped one."""
     g = torch.Generator().manual_seed(9)
     lens, starts = [300, 129, 5, 200], [40, 0, 7, 3]
